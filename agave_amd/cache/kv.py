@@ -29,7 +29,9 @@ from .pages import PAGE, CacheError, GroupKey, GroupPages, OutOfPages, SlotTable
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Fixed-size state of one memory: ``shape`` per sequence."""
+    """Fixed-size state of one memory: ``shape`` per sequence.  A mixer that keeps several
+    tensors states a dict ``{name: StateNeed}``; ``KVCache.state[memory]`` is then a dict of
+    tensors under the same names."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
 
@@ -71,29 +73,47 @@ class KVCache:
         self.v_store: List[Optional[torch.Tensor]] = []
         # bfloat16 groups whose head size is a multiple of 16 (up to 256) keep their pages in the
         # matrix cores' tile order; the others row by row
-        self.packed: List[bool] = [dtype == torch.bfloat16 and k.head_dim % 16 == 0 and k.head_dim <= 256
-                                   for k in self.group_keys]
+        for k in self.group_keys:
+            if k.layout not in ("tiles", "rows"):
+                raise CacheError(f"unknown page layout {k.layout!r}")
+            if k.layout == "tiles" and k.v_head_dim not in (None, k.head_dim):
+                raise CacheError("pages in tile order hold keys and values of one size; a mixer with narrower "
+                                 "values asks for the layout 'rows'")
+        self.packed: List[bool] = [k.layout == "tiles" and dtype == torch.bfloat16 and k.head_dim % 16 == 0
+                                   and k.head_dim <= 256 for k in self.group_keys]
         for key, mems, packed in zip(self.group_keys, members, self.packed):
             n = pages_per_group[key]
             hd_k = (key.head_dim + 31) // 32 * 32 if packed else key.head_dim
             if device is None:
                 self.k_store.append(None)
                 self.v_store.append(None)
+            elif key.layout == "rows":
+                vd = key.v_head_dim or key.head_dim
+                self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, key.head_dim), dtype=dtype, device=device))
+                self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, vd), dtype=dtype, device=device))
             else:
                 self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, hd_k), dtype=dtype, device=device))
                 self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, key.head_dim, PAGE), dtype=dtype, device=device))
         self.state_needs = dict(state_needs)
-        self.state: Dict[int, Optional[torch.Tensor]] = {}
+        self.state: Dict[int, object] = {}          # memory -> tensor [slots, ...], or {name: tensor} for several
+
+        def make(need: StateNeed):
+            return None if device is None else torch.zeros((max_slots,) + tuple(need.shape), dtype=need.dtype, device=device)
         for mem, need in state_needs.items():
-            self.state[mem] = None if device is None else torch.zeros((max_slots,) + tuple(need.shape), dtype=need.dtype, device=device)
+            self.state[mem] = {k: make(v) for k, v in need.items()} if isinstance(need, dict) else make(need)
 
     # ------------------------------------------------------------------ slots
     def alloc_slot(self) -> int:
         s = self.slots.alloc()
-        for t in self.state.values():
-            if t is not None:
-                t[s].zero_()
+        for t in self._state_tensors():
+            t[s].zero_()
         return s
+
+    def _state_tensors(self) -> List[torch.Tensor]:
+        out = []
+        for t in self.state.values():
+            out += [x for x in (t.values() if isinstance(t, dict) else [t]) if x is not None]
+        return out
 
     def free_slot(self, slot: int) -> None:
         self.slots.check(slot)
@@ -188,7 +208,7 @@ class KVCache:
 
     def bytes(self) -> int:
         total = 0
-        for t in self.k_store + self.v_store + list(self.state.values()):
+        for t in self.k_store + self.v_store + self._state_tensors():
             if t is not None:
                 total += t.numel() * t.element_size()
         return total

@@ -99,6 +99,29 @@ class GroupKey:
     window: Optional[int]      # None: all keys
     n_kv_heads: int
     head_dim: int
+    # A query sees only the keys of its own chunk of this many positions (chunks are counted from
+    # position 0 of the sequence); None: no chunks.  Pages of chunks that are over are given back.
+    chunk: Optional[int] = None
+    v_head_dim: Optional[int] = None   # size of a value head if it differs from the keys'
+    # "tiles": K [page, kv head, 64, head_dim] and V transposed [page, kv head, head_dim, 64], in the
+    # matrix cores' operand order where the sizes allow; "rows": K and V row by row,
+    # [page, kv head, 64, head_dim] and [page, kv head, 64, v_head_dim], never reordered
+    layout: str = "tiles"
+
+    @property
+    def reach(self) -> Optional[int]:
+        """Positions a query looks back over at most, itself included (None: all of them)."""
+        bounds = [b for b in (self.window, self.chunk) if b is not None]
+        return min(bounds) if bounds else None
+
+    def first_needed(self, length: int) -> int:
+        """The oldest position that a query at position >= ``length`` can still see."""
+        lo = 0
+        if self.window is not None:
+            lo = max(lo, length - self.window + 1)
+        if self.chunk is not None:
+            lo = max(lo, (length // self.chunk) * self.chunk)
+        return lo
 
 
 def pages_in_reach(window: Optional[int], max_context: int, max_new: int = 1) -> int:
@@ -131,14 +154,12 @@ class GroupPages:
 
     # the lowest page index that a query at position >= ``length`` can still reach
     def _first_needed(self, length: int) -> int:
-        if self.key.window is None:
-            return 0
-        return max(0, length - self.key.window + 1) // PAGE
+        return self.key.first_needed(length) // PAGE
 
     def table_width(self, max_context: int, max_new: int = 1) -> int:
         """Columns that a step's table needs at most for sequences up to ``max_context``
         positions when a step brings up to ``max_new`` tokens per sequence."""
-        return pages_in_reach(self.key.window, max_context, max_new)
+        return pages_in_reach(self.key.reach, max_context, max_new)
 
     def plan(self, slot: int, pos0: int, n_new: int) -> Tuple[int, List[int]]:
         """Make sure pages exist for positions ``pos0 .. pos0+n_new-1`` and return

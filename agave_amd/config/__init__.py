@@ -3,8 +3,9 @@ from .errors import ConfigError, UnsupportedArchitecture
 from .gemma3 import Gemma3Config
 from .registry import (Architecture, architectures, find_architecture, load_config,
                        read_config_json, register_architecture)
-from .spec import (AttentionSpec, FeedForwardSpec, GatedFfnSpec, LayerSpec, MixerSpec,
-                   ModelSpec, NormSpec, PositionSpec, RunEntry)
+from .rilenex import RilenexConfig
+from .spec import (AttentionSpec, DenseFfnSpec, FeedForwardSpec, GatedDeltaSpec, GatedFfnSpec, Hgrn2Spec, LayerSpec,
+                   MixerSpec, ModelSpec, NormSpec, ParallelMixerSpec, PositionSpec, RunEntry, TalkingAttentionSpec)
 
 register_architecture(Architecture(
     name=Gemma3Config.architecture,
@@ -12,8 +13,15 @@ register_architecture(Architecture(
     parse=Gemma3Config.from_dict,
     spec=lambda cfg, names=None: cfg.model_spec(names)))
 
+register_architecture(Architecture(
+    name=RilenexConfig.architecture,
+    model_types=("rilenex",),
+    parse=RilenexConfig.from_dict,
+    spec=lambda cfg, names=None: cfg.model_spec(names)))
+
 __all__ = [
-    "ConfigError", "UnsupportedArchitecture", "Gemma3Config", "Architecture", "architectures",
+    "ConfigError", "UnsupportedArchitecture", "Gemma3Config", "RilenexConfig", "Architecture", "architectures",
     "find_architecture", "load_config", "read_config_json", "register_architecture",
     "AttentionSpec", "FeedForwardSpec", "GatedFfnSpec", "LayerSpec", "MixerSpec", "ModelSpec",
-    "NormSpec", "PositionSpec", "RunEntry"]
+    "NormSpec", "PositionSpec", "RunEntry", "TalkingAttentionSpec", "GatedDeltaSpec", "Hgrn2Spec",
+    "ParallelMixerSpec", "DenseFfnSpec"]

@@ -41,7 +41,9 @@ def architectures() -> Tuple[str, ...]:
 def find_architecture(raw: dict) -> Architecture:
     """Pick the row by ``architectures[0]``, else by ``model_type`` (also inside
     ``text_config``)."""
-    names = raw.get("architectures") or []
+    names = list(raw.get("architectures") or [])
+    if isinstance(raw.get("architecture"), str):          # a single name instead of the list
+        names.append(raw["architecture"])
     for n in names:
         if n in _ARCHITECTURES:
             return _ARCHITECTURES[n]

@@ -30,6 +30,7 @@ class PositionSpec:
     rotary_dim: int = 0
     theta: float = 0.0
     factor: float = 1.0            # linear scaling: positions are divided by it
+    interleaved: bool = False      # the rotated pairs are (2i, 2i+1) instead of (i, i + rotary_dim/2)
 
 
 @dataclass(frozen=True)
@@ -60,8 +61,101 @@ class AttentionSpec(MixerSpec):
 
 
 @dataclass(frozen=True)
+class TalkingAttentionSpec(MixerSpec):
+    """Softmax attention whose heads' scores are mixed by a matrix before the softmax, with keys
+    and values of different sizes, an optional short convolution behind the projections, an
+    optional gate per head on the output, and keys limited to the query's own chunk of positions."""
+    hidden: int = 0
+    n_heads: int = 0
+    n_kv_heads: int = 0
+    head_dim: int = 0              # queries and keys
+    v_head_dim: int = 0            # values
+    scale: float = 1.0             # multiplies q.k
+    chunk: Optional[int] = None    # None: all earlier keys; C: keys j <= i with j // C == i // C
+    conv_taps: int = 0             # 0: no convolution
+    position: PositionSpec = PositionSpec("none")
+    q_norm: Optional[NormSpec] = None
+    k_norm: Optional[NormSpec] = None
+    q_proj: str = ""
+    k_proj: str = ""
+    v_proj: str = ""
+    o_proj: str = ""
+    q_conv: str = ""               # [channels, taps], the last column is the current token's
+    k_conv: str = ""
+    v_conv: str = ""
+    talk: str = ""                 # [heads, heads]: score_h <- sum_g talk[h, g] score_g; "": none
+    gate_proj: str = ""            # [heads, hidden]: head h's output times sigmoid(gate_proj x)_h; "": none
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec(MixerSpec):
+    """Delta rule with a decay per head and key channel (state [heads, head_dim, v_head_dim])."""
+    hidden: int = 0
+    n_heads: int = 0               # value heads, and states
+    n_kv_heads: int = 0            # query/key heads; head h reads head h // (n_heads / n_kv_heads)
+    head_dim: int = 0
+    v_head_dim: int = 0
+    conv_taps: int = 0
+    decay_rank: int = 0            # inner size of the decay's two projections
+    gate_rank: int = 0             # inner size of the output gate's two projections
+    norm_eps: float = 1e-5         # of the read-out's norm
+    unit_eps: float = 1e-6         # q and k become x / sqrt(sum(x^2) + unit_eps) per head
+    q_proj: str = ""
+    k_proj: str = ""
+    v_proj: str = ""
+    o_proj: str = ""
+    q_conv: str = ""
+    k_conv: str = ""
+    v_conv: str = ""
+    beta_proj: str = ""            # [heads, hidden]
+    decay_in: str = ""             # [decay_rank, hidden]
+    decay_out: str = ""            # [heads * head_dim, decay_rank]
+    decay_bias: str = ""           # [heads * head_dim]
+    decay_log: str = ""            # [heads]: the rate is exp of it
+    gate_in: str = ""              # [gate_rank, hidden]
+    gate_out: str = ""             # [heads * v_head_dim, gate_rank]
+    out_norm: str = ""             # [v_head_dim], shared by the heads
+
+
+@dataclass(frozen=True)
+class Hgrn2Spec(MixerSpec):
+    """Linear attention whose forget gate also sets what is written (state [heads, head_dim, v_head_dim])."""
+    hidden: int = 0
+    n_heads: int = 0
+    head_dim: int = 0
+    v_head_dim: int = 0
+    norm_eps: float = 1e-5
+    q_proj: str = ""
+    f_proj: str = ""
+    f_bias: str = ""
+    lower: str = ""                # [heads * head_dim]: the forget gate's lower bound
+    v_proj: str = ""
+    o_proj: str = ""
+    out_norm: str = ""             # [v_head_dim], shared by the heads
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec(MixerSpec):
+    """Mixers side by side on the same input; the result is the sum of ``scales[i] * branches[i]``."""
+    branches: Tuple[MixerSpec, ...] = ()
+    scales: Tuple[float, ...] = ()
+
+
+@dataclass(frozen=True)
 class FeedForwardSpec:
     kind: str
+
+
+@dataclass(frozen=True)
+class DenseFfnSpec(FeedForwardSpec):
+    """``W_down act(W_up x)``.  ``act_params`` names a small tensor of the activation's learned
+    numbers where it has some (xielu: two)."""
+    hidden: int = 0
+    intermediate: int = 0
+    activation: str = "gelu_tanh"
+    up_proj: str = ""
+    down_proj: str = ""
+    act_params: str = ""
 
 
 @dataclass(frozen=True)

@@ -487,6 +487,43 @@ extern "C" int agave_gated_act(int dtype, int act, const void* gate, long ldg, c
 }
 
 // (the tanh form of gelu under its older name)
+// ------------------------------------------------------------------ an activation on its own
+// out = act(x) for a feed-forward without a gate.  Activations 0 to 3 are the gate's; 4 is xIELU with
+// its two factors made by the host:  x > 0: ap x^2 + x/2;  x <= 0: an (exp(x) - 1 - x) + x/2.
+#define AGAVE_UNARY_ACTS 5
+template <typename T>
+__global__ void unary_act_kernel(const T* __restrict__ x, long ldx, T* __restrict__ out, long ldo, long total, int ff,
+                                 int act, float p0, float p1) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / ff;
+        const int c = (int)(idx % ff);
+        const float z = ld(x + r * ldx + c);
+        float y;
+        if (act == 4) y = z > 0.f ? fmaf(p0 * z, z, 0.5f * z) : fmaf(p1, expm1f(z) - z, 0.5f * z);
+        else y = gate_act(z, act);
+        st(out + r * ldo + c, y);
+    }
+}
+
+extern "C" int agave_unary_act(int dtype, int act, float p0, float p1, const void* x, long ldx, void* out, long ldo,
+                               int n_rows, int ff, hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && ff > 0, "unary_act: bad sizes rows=%d ff=%d", n_rows, ff);
+    AGAVE_CHECK(act >= 0 && act < AGAVE_UNARY_ACTS, "unary_act: unknown activation %d", act);
+    AGAVE_CHECK(x && out && ldx >= ff && ldo >= ff, "unary_act: bad buffers");
+    if (n_rows == 0) return 0;
+    const long total = (long)n_rows * ff;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == AGAVE_F32)
+        unary_act_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)x, ldx, (float*)out, ldo, total, ff, act, p0, p1);
+    else if (dtype == AGAVE_BF16)
+        unary_act_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)x, ldx, (bf16*)out, ldo, total, ff, act, p0, p1);
+    else
+        AGAVE_CHECK(false, "unary_act: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("unary_act");
+    return 0;
+}
+
 extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up, long ldu, void* out, long ldo,
                            int n_rows, int ff, hipStream_t stream) {
     return agave_gated_act(dtype, 0, gate, ldg, up, ldu, out, ldo, n_rows, ff, stream);

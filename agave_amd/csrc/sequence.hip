@@ -1,0 +1,600 @@
+// Kernels of the mixers that carry a state from token to token, and of the attention whose
+// heads talk to each other, for gfx950:
+//
+//   short causal convolution per channel, with the last taps - 1 inputs of a sequence as state;
+//   per-head RMS norm + rotation (pairs interleaved or split in halves) + cache write, for key and
+//     value heads of different sizes, pages stored row by row;
+//   attention over the paged cache with the heads' scores mixed by a matrix before the softmax,
+//     keys of the query's own chunk only (or all earlier keys), a gate per head;
+//   the gated linear recurrence S <- diag(a) S + k u^T, o = S^T q with u = beta (v - S^T k) (delta
+//     rule) or u = v (forget-gate form), the gates made inside;
+//   per-head RMS norm of the read-out with an optional elementwise sigmoid gate.
+//
+// Everything between the first product of a mixer and the rows its output product reads is 32-bit
+// here: projections arrive as float rows, state is float, angles are made in double.  T is the
+// element type of the cache pages and of the rows handed to the output product.
+#include "common_impl.h"
+#include <math.h>
+
+#define CONV_MAX_TAPS 8
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// ------------------------------------------------------------------ short causal convolution
+//   y[t][c] = act(sum_j w[c][j] * u[pos(t) - taps + 1 + j][c]),  zeros before the sequence's start.
+// Inputs older than the step's first token come from state[slot][taps - 1][C], which holds the
+// inputs at positions pos0 - taps + 1 .. pos0 - 1.  fused_update (every sequence brings one token):
+// the thread that owns (sequence, channel) also shifts the state; otherwise conv_state_kernel does
+// it afterwards, when no thread reads the old state any more.
+template <bool SILU>
+__global__ void short_conv_kernel(const float* __restrict__ u, long ldu, const float* __restrict__ w,
+                                  float* __restrict__ y, long ldy, float* __restrict__ state,
+                                  const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                  const int* __restrict__ pos0, const int* __restrict__ slots, int C, int taps,
+                                  int fused_update) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int t = blockIdx.y;
+    if (c >= C) return;
+    const int s = tok_seq[t], p = tok_pos[t], p0 = pos0[s];
+    float* st_c = state + ((size_t)slots[s] * (taps - 1)) * C + c;
+    float in[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        in[j] = 0.f;
+        if (j < taps) {
+            const int r = p - taps + 1 + j;                 // position of this tap's input
+            if (r >= p0) in[j] = u[(size_t)(t - (p - r)) * ldu + c];
+            else in[j] = st_c[(size_t)(r - (p0 - (taps - 1))) * C];
+        }
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j)
+        if (j < taps) acc = fmaf(w[(size_t)c * taps + j], in[j], acc);
+    y[(size_t)t * ldy + c] = SILU ? silu_f(acc) : acc;
+    if (fused_update) {
+#pragma unroll
+        for (int j = 1; j < CONV_MAX_TAPS; ++j)
+            if (j < taps) st_c[(size_t)(j - 1) * C] = in[j];
+    }
+}
+
+__global__ void conv_state_kernel(const float* __restrict__ u, long ldu, float* __restrict__ state,
+                                  const int* __restrict__ cu, const int* __restrict__ pos0,
+                                  const int* __restrict__ slots, int C, int taps) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int s = blockIdx.y;
+    if (c >= C) return;
+    const int r0 = cu[s], n = cu[s + 1] - r0;
+    float* st_c = state + ((size_t)slots[s] * (taps - 1)) * C + c;
+    float keep[CONV_MAX_TAPS];
+#pragma unroll
+    for (int i = 0; i < CONV_MAX_TAPS - 1; ++i) {
+        keep[i] = 0.f;
+        if (i < taps - 1) {
+            const int back = taps - 1 - i;                  // the input `back` positions before the new end
+            if (back <= n) keep[i] = u[(size_t)(r0 + n - back) * ldu + c];
+            else keep[i] = st_c[(size_t)(i + n) * C];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < CONV_MAX_TAPS - 1; ++i)
+        if (i < taps - 1) st_c[(size_t)i * C] = keep[i];
+}
+
+extern "C" int agave_short_conv(const float* u, long ldu, const float* w, float* y, long ldy, float* state,
+                                const int* tok_seq, const int* tok_pos, const int* cu, const int* pos0,
+                                const int* slots, int n_tokens, int n_seqs, int C, int taps, int silu,
+                                int one_token_each, hipStream_t stream) {
+    AGAVE_CHECK(n_tokens >= 0 && n_seqs >= 0 && C > 0, "short_conv: bad sizes N=%d B=%d C=%d", n_tokens, n_seqs, C);
+    AGAVE_CHECK(taps >= 2 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (2 to %d are supported)", taps, CONV_MAX_TAPS);
+    AGAVE_CHECK(ldu >= C && ldy >= C, "short_conv: a row stride is below %d", C);
+    AGAVE_CHECK(u && w && y && state && tok_seq && tok_pos && cu && pos0 && slots, "short_conv: null buffer");
+    AGAVE_CHECK(u != y, "short_conv: the convolution is not done in place");
+    AGAVE_CHECK(n_tokens < 65536 * 16, "short_conv: too many tokens");
+    if (n_tokens == 0) return 0;
+    const int threads = C >= 256 ? 256 : 64;
+    const dim3 grid((C + threads - 1) / threads, n_tokens);
+    if (silu)
+        short_conv_kernel<true><<<grid, threads, 0, stream>>>(u, ldu, w, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
+    else
+        short_conv_kernel<false><<<grid, threads, 0, stream>>>(u, ldu, w, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
+    AGAVE_LAUNCH_CHECK("short_conv");
+    if (!one_token_each) {
+        conv_state_kernel<<<dim3((C + threads - 1) / threads, n_seqs), threads, 0, stream>>>(u, ldu, state, cu, pos0, slots, C, taps);
+        AGAVE_LAUNCH_CHECK("conv_state");
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------ head norm + rotation + cache rows
+// A wave per (token, head).  Heads 0 .. nh-1 are queries (written to q_out as float rows), the next
+// nkv are keys (into k_pages [page][kv head][64][dk]) and the last nkv values (copied into v_pages
+// [page][kv head][64][dv]).  Norm: x * rsqrt(mean(x^2) + eps) * gain (gain may be null).  Rotation of
+// the first 2 * rot_half elements: interleaved pairs (2i, 2i+1) or halves (i, i + rot_half); the pair
+// (a, b) at position p becomes (a cos - b sin, b cos + a sin), angle p * freq[i] made in double.
+template <typename T>
+__global__ __launch_bounds__(64) void head_norm_rope_rows_kernel(
+    const float* __restrict__ q, long ldq, const float* __restrict__ k, long ldk, const float* __restrict__ v, long ldv,
+    float* __restrict__ q_out, long ldqo, const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+    float eps_q, float eps_k, int norm_q, int norm_k, const double* __restrict__ freq, int rot_half, int interleaved,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    const int* __restrict__ table, int width, const int* __restrict__ base, int n_pages, int nh, int nkv, int dk, int dv) {
+    const int per_tok = nh + 2 * nkv;
+    const int t = blockIdx.x / per_tok, head = blockIdx.x % per_tok;
+    const int lane = threadIdx.x;
+    const int p = tok_pos[t];
+    long row = -1;                                          // row of the cache this head is written to
+    if (head >= nh) {
+        const int b = tok_seq[t];
+        const int col = p / AGAVE_PAGE - base[b];
+        int pg = (col >= 0 && col < width) ? table[(size_t)b * width + col] : -1;
+        if (pg < 0 || pg >= n_pages) return;               // the planner never leaves such a hole
+        const int kvh = head >= nh + nkv ? head - nh - nkv : head - nh;
+        row = ((long)pg * nkv + kvh) * AGAVE_PAGE + (p % AGAVE_PAGE);
+    }
+    if (head >= nh + nkv) {
+        const float* x = v + (size_t)t * ldv + (size_t)(head - nh - nkv) * dv;
+        T* o = v_pages + (size_t)row * dv;
+        for (int d = lane; d < dv; d += 64) st(o + d, x[d]);
+        return;
+    }
+    const bool is_q = head < nh;
+    const float* x = is_q ? q + (size_t)t * ldq + (size_t)head * dk : k + (size_t)t * ldk + (size_t)(head - nh) * dk;
+    const float* gain = is_q ? q_gain : k_gain;
+    const bool normed = is_q ? norm_q : norm_k;
+    float inv = 1.f;
+    if (normed) {
+        float ss = 0.f;
+        for (int d = lane; d < dk; d += 64) ss = fmaf(x[d], x[d], ss);
+        ss = wave_sum(ss);
+        inv = 1.0f / sqrtf(ss / (float)dk + (is_q ? eps_q : eps_k));
+    }
+    for (int d = lane; d < dk; d += 64) {
+        float val = x[d] * inv * (gain ? gain[d] : 1.f);
+        if (d < 2 * rot_half) {
+            int fi, other;
+            bool first;
+            if (interleaved) { fi = d >> 1; other = d ^ 1; first = !(d & 1); }
+            else { fi = d < rot_half ? d : d - rot_half; other = d < rot_half ? d + rot_half : d - rot_half; first = d < rot_half; }
+            const float oth = x[other] * inv * (gain ? gain[other] : 1.f);
+            const double ang = (double)p * freq[fi];
+            const float c = (float)cos(ang), s = (float)sin(ang);
+            val = first ? val * c - oth * s : val * c + oth * s;
+        }
+        if (is_q) q_out[(size_t)t * ldqo + (size_t)head * dk + d] = val;
+        else st(k_pages + (size_t)row * dk + d, val);
+    }
+}
+
+extern "C" int agave_head_norm_rope_rows(int dtype, const float* q, long ldq, const float* k, long ldk, const float* v,
+                                         long ldv, float* q_out, long ldqo, const float* q_gain, const float* k_gain,
+                                         float eps_q, float eps_k, int norm_q, int norm_k, const double* freq,
+                                         int rot_half, int interleaved, const int* tok_seq, const int* tok_pos,
+                                         void* k_pages, void* v_pages, const int* table, int width, const int* base,
+                                         int n_pages, int N, int nh, int nkv, int dk, int dv, hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && nh >= 0 && nkv >= 0 && dk > 0 && dv > 0, "head_norm_rope_rows: bad sizes N=%d nh=%d nkv=%d dk=%d dv=%d", N, nh, nkv, dk, dv);
+    AGAVE_CHECK(rot_half >= 0 && 2 * rot_half <= dk, "head_norm_rope_rows: %d rotated elements exceed the head's %d", 2 * rot_half, dk);
+    AGAVE_CHECK(rot_half == 0 || freq, "head_norm_rope_rows: rotation without a frequency table");
+    AGAVE_CHECK(nh == 0 || (q && q_out && ldq >= (long)nh * dk && ldqo >= (long)nh * dk), "head_norm_rope_rows: bad q buffers");
+    AGAVE_CHECK(nkv == 0 || (k && v && k_pages && v_pages && table && base && width > 0 && n_pages > 0 &&
+                             ldk >= (long)nkv * dk && ldv >= (long)nkv * dv), "head_norm_rope_rows: bad k/v buffers");
+    AGAVE_CHECK(tok_seq && tok_pos, "head_norm_rope_rows: null token tables");
+    AGAVE_CHECK((long)N * (nh + 2 * nkv) < 2147483647L, "head_norm_rope_rows: too many rows");
+    if (N == 0 || nh + nkv == 0) return 0;
+    const int grid = N * (nh + 2 * nkv);
+    if (dtype == AGAVE_F32)
+        head_norm_rope_rows_kernel<float><<<grid, 64, 0, stream>>>(q, ldq, k, ldk, v, ldv, q_out, ldqo, q_gain, k_gain, eps_q, eps_k,
+            norm_q, norm_k, freq, rot_half, interleaved, tok_seq, tok_pos, (float*)k_pages, (float*)v_pages, table, width, base,
+            n_pages, nh, nkv, dk, dv);
+    else if (dtype == AGAVE_BF16)
+        head_norm_rope_rows_kernel<bf16><<<grid, 64, 0, stream>>>(q, ldq, k, ldk, v, ldv, q_out, ldqo, q_gain, k_gain, eps_q, eps_k,
+            norm_q, norm_k, freq, rot_half, interleaved, tok_seq, tok_pos, (bf16*)k_pages, (bf16*)v_pages, table, width, base,
+            n_pages, nh, nkv, dk, dv);
+    else
+        AGAVE_CHECK(false, "head_norm_rope_rows: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("head_norm_rope_rows");
+    return 0;
+}
+
+// ------------------------------------------------------------------ attention with talking heads
+// A workgroup per query token, all heads at once (the mixing needs every head's score of a key):
+//   raw[g][j]  = scale * q_g . k_j            (key head of g: g / (nh / nkv))
+//   s[h][j]    = sum_g talk[h][g] raw[g][j]   (talk null: s = raw)
+//   w[h][.]    = softmax over the visible keys j: j <= p, and j >= floor(p / chunk) * chunk if chunk > 0
+//   out[h]     = sigmoid(gate[h]) * out_scale * sum_j w[h][j] v_j
+// Keys come in tiles of 64 with a running maximum and sum per head.  Dynamic LDS:
+//   qs[nh*dk] raw[nh*64] mix[nh*64] talk[nh*nh] m[nh] l[nh] alpha[nh] pg[64]
+#define TALK_ACC 16
+template <typename T>
+__global__ __launch_bounds__(256) void talk_attention_kernel(
+    const float* __restrict__ q, long ldq, const float* __restrict__ gate, long ldg, T* __restrict__ out, long ldo,
+    const T* __restrict__ k_pages, const T* __restrict__ v_pages, const int* __restrict__ table, int width,
+    const int* __restrict__ base, int n_pages, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+    const float* __restrict__ talk, int nh, int nkv, int dk, int dv, float scale, int chunk, float out_scale) {
+    extern __shared__ float lds[];
+    float* qs = lds;
+    float* raw = qs + (size_t)nh * dk;
+    float* mix = raw + (size_t)nh * 64;
+    float* tk = mix + (size_t)nh * 64;
+    float* m_run = tk + (size_t)nh * nh;
+    float* l_run = m_run + nh;
+    float* alpha = l_run + nh;
+    int* pg = reinterpret_cast<int*>(alpha + nh);
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int t = blockIdx.x;
+    const int b = tok_seq[t], p = tok_pos[t];
+    const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
+    const int rep = nh / nkv;
+    const int pbase = base[b];
+
+    for (int i = tid; i < nh * dk; i += 256) qs[i] = q[(size_t)t * ldq + i];
+    if (talk)
+        for (int i = tid; i < nh * nh; i += 256) tk[i] = talk[i];
+    for (int i = tid; i < nh; i += 256) { m_run[i] = -INFINITY; l_run[i] = 0.f; }
+    float acc[TALK_ACC];
+#pragma unroll
+    for (int a = 0; a < TALK_ACC; ++a) acc[a] = 0.f;
+    __syncthreads();
+
+    for (int j0 = lo; j0 <= p; j0 += 64) {
+        const int nk = p - j0 + 1 < 64 ? p - j0 + 1 : 64;
+        if (tid < 64) {
+            int id = -1;
+            const int j = j0 + tid;
+            if (tid < nk) {
+                const int col = j / AGAVE_PAGE - pbase;
+                if (col >= 0 && col < width) id = table[(size_t)b * width + col];
+                if (id >= n_pages) id = -1;
+            }
+            pg[tid] = id;
+        }
+        __syncthreads();
+        // raw scores: lane = key, the waves share the heads
+        {
+            const int j = j0 + lane;
+            const int id = pg[lane];
+            for (int h = wv; h < nh; h += 4) {
+                float s = 0.f;
+                if (id >= 0) {
+                    const T* kr = k_pages + (((size_t)id * nkv + h / rep) * AGAVE_PAGE + (j % AGAVE_PAGE)) * dk;
+                    const float* qh = qs + (size_t)h * dk;
+                    float dot = 0.f;
+                    for (int d = 0; d < dk; ++d) dot = fmaf(qh[d], ld(kr + d), dot);
+                    s = dot * scale;
+                }
+                raw[h * 64 + lane] = s;
+            }
+        }
+        __syncthreads();
+        // mixing, then each head's running maximum and sum (a wave per head in turn)
+        for (int h = wv; h < nh; h += 4) {
+            float s;
+            if (talk) {
+                s = 0.f;
+                for (int g = 0; g < nh; ++g) s = fmaf(tk[h * nh + g], raw[g * 64 + lane], s);
+            } else {
+                s = raw[h * 64 + lane];
+            }
+            const bool valid = lane < nk && pg[lane] >= 0;
+            if (!valid) s = -INFINITY;
+            const float tmax = wave_max(s);
+            const float m_old = m_run[h];
+            const float m_new = fmaxf(m_old, tmax);
+            const float al = (m_old == -INFINITY) ? 0.f : expf(m_old - m_new);
+            const float pr = valid ? expf(s - m_new) : 0.f;
+            mix[h * 64 + lane] = pr;
+            const float sum = wave_sum(pr);
+            if (lane == 0) {
+                m_run[h] = m_new;
+                l_run[h] = l_run[h] * al + sum;
+                alpha[h] = al;
+            }
+        }
+        __syncthreads();
+        // weighted sum of the values: a thread per (head, value element)
+#pragma unroll
+        for (int a = 0; a < TALK_ACC; ++a) {
+            const int idx = tid + a * 256;
+            if (idx < nh * dv) {
+                const int h = idx / dv, e = idx % dv;
+                const int kvh = h / rep;
+                float sum = 0.f;
+                for (int r = 0; r < nk; ++r) {
+                    const int id = pg[r];
+                    if (id < 0) continue;
+                    const T* vr = v_pages + (((size_t)id * nkv + kvh) * AGAVE_PAGE + ((j0 + r) % AGAVE_PAGE)) * dv;
+                    sum = fmaf(mix[h * 64 + r], ld(vr + e), sum);
+                }
+                acc[a] = acc[a] * alpha[h] + sum;
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int a = 0; a < TALK_ACC; ++a) {
+        const int idx = tid + a * 256;
+        if (idx < nh * dv) {
+            const int h = idx / dv;
+            const float l = l_run[h];
+            float o = l > 0.f ? acc[a] / l : 0.f;
+            if (gate) o *= sigmoid_f(gate[(size_t)t * ldg + h]);
+            st(out + (size_t)t * ldo + idx, o * out_scale);
+        }
+    }
+}
+
+extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const float* gate, long ldg, void* out, long ldo,
+                                    const void* k_pages, const void* v_pages, const int* table, int width,
+                                    const int* base, int n_pages, const int* tok_seq, const int* tok_pos,
+                                    const float* talk, int N, int nh, int nkv, int dk, int dv, float scale, int chunk,
+                                    float out_scale, hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "talk_attention: bad sizes N=%d nh=%d nkv=%d dk=%d dv=%d", N, nh, nkv, dk, dv);
+    AGAVE_CHECK(nh % nkv == 0, "talk_attention: %d query heads are not a multiple of %d key heads", nh, nkv);
+    AGAVE_CHECK((long)nh * dv <= 256 * TALK_ACC, "talk_attention: heads x value size %ld exceeds %d", (long)nh * dv, 256 * TALK_ACC);
+    AGAVE_CHECK(ldq >= (long)nh * dk && ldo >= (long)nh * dv && (!gate || ldg >= nh), "talk_attention: a row stride is too small");
+    AGAVE_CHECK(chunk >= 0, "talk_attention: negative chunk");
+    AGAVE_CHECK(q && out && k_pages && v_pages && table && base && tok_seq && tok_pos && width > 0 && n_pages > 0,
+                "talk_attention: null buffer or empty table");
+    const size_t lds = ((size_t)nh * dk + 2 * (size_t)nh * 64 + (size_t)nh * nh + 3 * (size_t)nh + 64) * sizeof(float);
+    AGAVE_CHECK(lds <= 64 * 1024, "talk_attention: %d heads of size %d need %zu bytes of LDS (64 KB are there)", nh, dk, lds);
+    if (N == 0) return 0;
+    if (dtype == AGAVE_F32)
+        talk_attention_kernel<float><<<N, 256, lds, stream>>>(q, ldq, gate, ldg, (float*)out, ldo, (const float*)k_pages,
+            (const float*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale);
+    else if (dtype == AGAVE_BF16)
+        talk_attention_kernel<bf16><<<N, 256, lds, stream>>>(q, ldq, gate, ldg, (bf16*)out, ldo, (const bf16*)k_pages,
+            (const bf16*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale);
+    else
+        AGAVE_CHECK(false, "talk_attention: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("talk_attention");
+    return 0;
+}
+
+// ------------------------------------------------------------------ gated linear recurrence
+// Per sequence and head a state S [dk][dv] of floats, advanced token by token:
+//     S <- diag(a) S;   u = beta (v - S^T k)  [delta]  or  u = v  [forget gate];   S <- S + k u^T;   o = S^T q
+// so the read-out sees the token's own write.  A column of S (one value element) never meets
+// another, so a workgroup owns 64 columns and four lanes share a column's dk rows (R each).
+// The gates of 16 tokens at a time are made by the whole workgroup into LDS, then the 16 tokens
+// run one after another:
+//   delta:   q, k: unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times dk^-1/2; key head of h is
+//            h / (nh / nkv);  a = exp(-exp(A_log[h]) * softplus(dt[h][d] + dt_bias[h][d]));  beta = sigmoid(b[h])
+//   forget:  q = silu(q);  f = low + (1 - low) sigmoid(f_in + f_bias);  a = f, k = 1 - f
+#define REC_DELTA 0
+#define REC_FORGET 1
+#define REC_TOKENS 16
+
+struct RecurrenceArgs {
+    const float* q; long ldq;          // delta: [N, nkv*dk]; forget: [N, nh*dk]
+    const float* k; long ldk;          // delta: keys [N, nkv*dk]; forget: the gate's input [N, nh*dk]
+    const float* v; long ldv;          // [N, nh*dv]
+    const float* dt; long lddt;        // delta: [N, nh*dk]
+    const float* b; long ldb;          // delta: [N, nh]
+    const float* a_log;                // delta: [nh]
+    const float* dt_bias;              // delta: [nh*dk]
+    const float* low;                  // forget: [nh*dk]
+    const float* f_bias;               // forget: [nh*dk] or null
+    float* o; long ldo;                // [N, nh*dv]
+    float* state;                      // [slots][nh][dk][dv]
+    const int* cu; const int* slots;
+    int nh, nkv, dk, dv;
+    float unit_eps;                    // delta: inside the root of the unit vectors
+};
+
+__device__ __forceinline__ float quad_sum(float v) {
+    v += dpp_get<0xB1, 0xF>(0.f, v);
+    v += dpp_get<0x4E, 0xF>(0.f, v);
+    return v;
+}
+
+template <int MODE, int R>
+__global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs A) {
+    constexpr int DP = 4 * R;                               // padded rows
+    __shared__ __attribute__((aligned(16))) float sa[REC_TOKENS][DP];
+    __shared__ __attribute__((aligned(16))) float sk[REC_TOKENS][DP];
+    __shared__ __attribute__((aligned(16))) float sq[REC_TOKENS][DP];
+    __shared__ float sv[REC_TOKENS][64];
+    __shared__ float sbeta[REC_TOKENS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int vl = tid >> 2, ds = tid & 3;
+    const int h = blockIdx.y, s = blockIdx.z;
+    const int col = blockIdx.x * 64 + vl;
+    const int dk = A.dk, dv = A.dv;
+    const int r0 = A.cu[s], r1 = A.cu[s + 1];
+    float* S_g = A.state + (((size_t)A.slots[s] * A.nh + h) * dk) * dv;
+
+    float S[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int d = ds * R + i;
+        S[i] = (d < dk && col < dv) ? S_g[(size_t)d * dv + col] : 0.f;
+    }
+    const int kvh = MODE == REC_DELTA ? h / (A.nh / A.nkv) : h;
+
+    for (int tb = r0; tb < r1; tb += REC_TOKENS) {
+        const int nt = r1 - tb < REC_TOKENS ? r1 - tb : REC_TOKENS;
+        __syncthreads();                                    // the tokens before are done with the LDS
+        // ---- the gates of these tokens: a wave per token in turn
+        for (int tt = wv; tt < nt; tt += 4) {
+            const size_t row = (size_t)(tb + tt);
+            if (MODE == REC_DELTA) {
+                const float* qr = A.q + row * A.ldq + (size_t)kvh * dk;
+                const float* kr = A.k + row * A.ldk + (size_t)kvh * dk;
+                float qq = 0.f, kk = 0.f;
+                for (int d = lane; d < dk; d += 64) { qq = fmaf(qr[d], qr[d], qq); kk = fmaf(kr[d], kr[d], kk); }
+                qq = wave_sum(qq);
+                kk = wave_sum(kk);
+                const float qi = 1.0f / sqrtf(qq + A.unit_eps) / sqrtf((float)dk), ki = 1.0f / sqrtf(kk + A.unit_eps);
+                const float ea = expf(A.a_log[h]);
+                for (int d = lane; d < DP; d += 64) {
+                    float a = 0.f, kx = 0.f, qx = 0.f;
+                    if (d < dk) {
+                        const float x = A.dt[row * A.lddt + (size_t)h * dk + d] + A.dt_bias[(size_t)h * dk + d];
+                        a = expf(-ea * softplus_f(x));
+                        kx = kr[d] * ki;
+                        qx = qr[d] * qi;
+                    }
+                    sa[tt][d] = a; sk[tt][d] = kx; sq[tt][d] = qx;
+                }
+                if (lane == 0) sbeta[tt] = sigmoid_f(A.b[row * A.ldb + h]);
+            } else {
+                for (int d = lane; d < DP; d += 64) {
+                    float a = 0.f, kx = 0.f, qx = 0.f;
+                    if (d < dk) {
+                        const size_t c = (size_t)h * dk + d;
+                        const float lw = A.low[c];
+                        const float f = lw + (1.f - lw) * sigmoid_f(A.k[row * A.ldk + c] + (A.f_bias ? A.f_bias[c] : 0.f));
+                        a = f;
+                        kx = 1.f - f;
+                        qx = silu_f(A.q[row * A.ldq + c]);
+                    }
+                    sa[tt][d] = a; sk[tt][d] = kx; sq[tt][d] = qx;
+                }
+            }
+            const int c = blockIdx.x * 64 + lane;
+            sv[tt][lane] = c < dv ? A.v[row * A.ldv + (size_t)h * dv + c] : 0.f;
+        }
+        __syncthreads();
+        // ---- the tokens, one after another
+        for (int tt = 0; tt < nt; ++tt) {
+            const float4* a4 = reinterpret_cast<const float4*>(&sa[tt][ds * R]);
+            const float4* k4 = reinterpret_cast<const float4*>(&sk[tt][ds * R]);
+            const float4* q4 = reinterpret_cast<const float4*>(&sq[tt][ds * R]);
+            float kreg[R];
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < R / 4; ++i) {
+                const float4 a = a4[i], k = k4[i];
+                kreg[4 * i] = k.x; kreg[4 * i + 1] = k.y; kreg[4 * i + 2] = k.z; kreg[4 * i + 3] = k.w;
+                S[4 * i] *= a.x; S[4 * i + 1] *= a.y; S[4 * i + 2] *= a.z; S[4 * i + 3] *= a.w;
+                if (MODE == REC_DELTA) {
+                    dot = fmaf(S[4 * i], k.x, dot); dot = fmaf(S[4 * i + 1], k.y, dot);
+                    dot = fmaf(S[4 * i + 2], k.z, dot); dot = fmaf(S[4 * i + 3], k.w, dot);
+                }
+            }
+            float u = sv[tt][vl];
+            if (MODE == REC_DELTA) u = sbeta[tt] * (u - quad_sum(dot));
+            float o = 0.f;
+#pragma unroll
+            for (int i = 0; i < R / 4; ++i) {
+                const float4 qv = q4[i];
+                S[4 * i] = fmaf(kreg[4 * i], u, S[4 * i]); S[4 * i + 1] = fmaf(kreg[4 * i + 1], u, S[4 * i + 1]);
+                S[4 * i + 2] = fmaf(kreg[4 * i + 2], u, S[4 * i + 2]); S[4 * i + 3] = fmaf(kreg[4 * i + 3], u, S[4 * i + 3]);
+                o = fmaf(S[4 * i], qv.x, o); o = fmaf(S[4 * i + 1], qv.y, o);
+                o = fmaf(S[4 * i + 2], qv.z, o); o = fmaf(S[4 * i + 3], qv.w, o);
+            }
+            o = quad_sum(o);
+            if (ds == 0 && col < dv) A.o[(size_t)(tb + tt) * A.ldo + (size_t)h * dv + col] = o;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int d = ds * R + i;
+        if (d < dk && col < dv) S_g[(size_t)d * dv + col] = S[i];
+    }
+}
+
+template <int MODE>
+static int launch_recurrence(const RecurrenceArgs& A, int n_seqs, hipStream_t stream) {
+    const dim3 grid((A.dv + 63) / 64, A.nh, n_seqs);
+    if (A.dk <= 32) gated_recurrence_kernel<MODE, 8><<<grid, 256, 0, stream>>>(A);
+    else if (A.dk <= 64) gated_recurrence_kernel<MODE, 16><<<grid, 256, 0, stream>>>(A);
+    else if (A.dk <= 128) gated_recurrence_kernel<MODE, 32><<<grid, 256, 0, stream>>>(A);
+    else gated_recurrence_kernel<MODE, 64><<<grid, 256, 0, stream>>>(A);
+    AGAVE_LAUNCH_CHECK("gated_recurrence");
+    return 0;
+}
+
+extern "C" int agave_gated_recurrence(int mode, const float* q, long ldq, const float* k, long ldk, const float* v, long ldv,
+                                      const float* dt, long lddt, const float* b, long ldb, const float* a_log,
+                                      const float* dt_bias, const float* low, const float* f_bias, float* o, long ldo,
+                                      float* state, const int* cu, const int* slots, int n_seqs, int nh, int nkv, int dk,
+                                      int dv, float unit_eps, hipStream_t stream) {
+    AGAVE_CHECK(mode == REC_DELTA || mode == REC_FORGET, "gated_recurrence: unknown mode %d", mode);
+    AGAVE_CHECK(n_seqs >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "gated_recurrence: bad sizes B=%d nh=%d nkv=%d dk=%d dv=%d", n_seqs, nh, nkv, dk, dv);
+    AGAVE_CHECK(dk <= 256, "gated_recurrence: %d key channels a head (up to 256 are supported)", dk);
+    AGAVE_CHECK(nh % nkv == 0, "gated_recurrence: %d heads are not a multiple of %d key heads", nh, nkv);
+    AGAVE_CHECK(q && k && v && o && state && cu && slots, "gated_recurrence: null buffer");
+    AGAVE_CHECK(ldv >= (long)nh * dv && ldo >= (long)nh * dv, "gated_recurrence: a row stride is too small");
+    AGAVE_CHECK(n_seqs < 65536 && nh < 65536, "gated_recurrence: too many sequences or heads");
+    if (mode == REC_DELTA) {
+        AGAVE_CHECK(dt && b && a_log && dt_bias, "gated_recurrence: the delta rule needs dt, b, A_log and dt_bias");
+        AGAVE_CHECK(ldq >= (long)nkv * dk && ldk >= (long)nkv * dk && lddt >= (long)nh * dk && ldb >= nh, "gated_recurrence: a row stride is too small");
+    } else {
+        AGAVE_CHECK(low, "gated_recurrence: the forget gate needs its lower bound");
+        AGAVE_CHECK(nkv == nh && ldq >= (long)nh * dk && ldk >= (long)nh * dk, "gated_recurrence: the forget-gate form has a gate per head");
+    }
+    if (n_seqs == 0) return 0;
+    RecurrenceArgs A{q, ldq, k, ldk, v, ldv, dt, lddt, b, ldb, a_log, dt_bias, low, f_bias, o, ldo, state, cu, slots, nh, nkv, dk, dv, unit_eps};
+    return mode == REC_DELTA ? launch_recurrence<REC_DELTA>(A, n_seqs, stream) : launch_recurrence<REC_FORGET>(A, n_seqs, stream);
+}
+
+// ------------------------------------------------------------------ read-out norm with a gate
+//   out[t][h][e] = o[t][h][e] * rsqrt(mean_e(o[t][h]^2) + eps) * w[e] * (gate ? sigmoid(gate[t][h][e]) : 1) * out_scale
+template <typename T>
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(const float* __restrict__ o, long ldo_in, const float* __restrict__ w,
+                                                            const float* __restrict__ gate, long ldg, T* __restrict__ out,
+                                                            long ldo, int nh, int dv, float eps, float out_scale) {
+    const int t = blockIdx.x / nh, h = blockIdx.x % nh, lane = threadIdx.x;
+    const float* x = o + (size_t)t * ldo_in + (size_t)h * dv;
+    float ss = 0.f;
+    for (int e = lane; e < dv; e += 64) ss = fmaf(x[e], x[e], ss);
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+    for (int e = lane; e < dv; e += 64) {
+        float y = x[e] * inv * w[e];
+        if (gate) y *= sigmoid_f(gate[(size_t)t * ldg + (size_t)h * dv + e]);
+        st(out + (size_t)t * ldo + (size_t)h * dv + e, y * out_scale);
+    }
+}
+
+extern "C" int agave_head_norm_gate(int dtype, const float* o, long ldo_in, const float* w, const float* gate, long ldg,
+                                    void* out, long ldo, int N, int nh, int dv, float eps, float out_scale, hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && nh > 0 && dv > 0, "head_norm_gate: bad sizes N=%d nh=%d dv=%d", N, nh, dv);
+    AGAVE_CHECK(o && w && out && ldo_in >= (long)nh * dv && ldo >= (long)nh * dv && (!gate || ldg >= (long)nh * dv), "head_norm_gate: bad buffers");
+    AGAVE_CHECK((long)N * nh < 2147483647L, "head_norm_gate: too many rows");
+    if (N == 0) return 0;
+    if (dtype == AGAVE_F32)
+        head_norm_gate_kernel<float><<<N * nh, 64, 0, stream>>>(o, ldo_in, w, gate, ldg, (float*)out, ldo, nh, dv, eps, out_scale);
+    else if (dtype == AGAVE_BF16)
+        head_norm_gate_kernel<bf16><<<N * nh, 64, 0, stream>>>(o, ldo_in, w, gate, ldg, (bf16*)out, ldo, nh, dv, eps, out_scale);
+    else
+        AGAVE_CHECK(false, "head_norm_gate: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("head_norm_gate");
+    return 0;
+}
+
+// ------------------------------------------------------------------ a weighted sum of two branches
+//   out = sa * a + sb * b, summed in 32-bit (for mixers that run side by side and cannot share an output product)
+template <typename T>
+__global__ void scaled_sum_kernel(const T* __restrict__ a, long lda, float sa, const T* __restrict__ b, long ldb, float sb,
+                                  T* __restrict__ out, long ldo, long total, int cols) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / cols;
+        const int c = (int)(idx % cols);
+        st(out + r * ldo + c, sa * ld(a + r * lda + c) + sb * ld(b + r * ldb + c));
+    }
+}
+
+extern "C" int agave_scaled_sum(int dtype, const void* a, long lda, float sa, const void* b, long ldb, float sb, void* out,
+                                long ldo, int rows, int cols, hipStream_t stream) {
+    AGAVE_CHECK(rows >= 0 && cols > 0 && lda >= cols && ldb >= cols && ldo >= cols, "scaled_sum: bad sizes rows=%d cols=%d", rows, cols);
+    AGAVE_CHECK(a && b && out, "scaled_sum: null buffer");
+    if (rows == 0) return 0;
+    const long total = (long)rows * cols;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == AGAVE_F32)
+        scaled_sum_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)a, lda, sa, (const float*)b, ldb, sb, (float*)out, ldo, total, cols);
+    else if (dtype == AGAVE_BF16)
+        scaled_sum_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)a, lda, sa, (const bf16*)b, ldb, sb, (bf16*)out, ldo, total, cols);
+    else
+        AGAVE_CHECK(false, "scaled_sum: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("scaled_sum");
+    return 0;
+}

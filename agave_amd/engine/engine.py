@@ -82,11 +82,14 @@ class Engine:
         # what this element type needs is compiled now, side by side, rather than one library
         # after the other as the first step meets them (a fresh checkout's first run)
         from ..ops import library
-        needed = ["elementwise", "gemm", "attention_plain"]
+        from ..parts import mixer_libraries
+        needed = ["elementwise", "gemm"]
         if will_sample:                    # (a caller that only wants logits, like trace replay, builds no sampling kernels)
             needed.append("sampling")
         if self.dtype == torch.bfloat16:
-            needed += ["gemm_mfma", "attention_mfma"]
+            needed.append("gemm_mfma")
+        for layer in spec.layers:          # what the model's own mixers run on, and no more
+            needed += sorted(mixer_libraries(layer.mixer, self.dtype) - set(needed))
         library.ensure_built(needed)
         self.workspace = Workspace(self.device)
         self.env = BuildEnv(self.dtype, self.device, self.workspace, keep_stored_precision=bool(keep_stored_precision))
@@ -109,7 +112,7 @@ class Engine:
         pages: Dict[GroupKey, int] = {}
         for key in set(kv_needs.values()):
             # what max_slots sequences can hold at most; fewer if the caller bounds the live positions
-            pages[key] = pool_pages(key.window, max_slots, self.max_context, self.max_piece)
+            pages[key] = pool_pages(key.reach, max_slots, self.max_context, self.max_piece)
             if cache_tokens is not None:
                 pages[key] = min(pages[key], max(1, (int(cache_tokens) + PAGE - 1) // PAGE))
         self.cache = KVCache(kv_needs, self.model.state_needs(), max_slots, pages, self.dtype, self.device,
@@ -133,7 +136,7 @@ class Engine:
         arch = find_architecture(raw)
         cfg = arch.parse(raw)
         ckpt = Checkpoint(model_dir)
-        spec = arch.spec(cfg, ckpt.names())
+        spec = arch.spec(cfg, {n: tuple(ckpt.shape(n)) for n in ckpt.names()})     # names, with their shapes
         weights = WeightSource(ckpt, tensor_needs(spec), spec.tensor_scope)
         return cls(spec, weights, config=cfg, **kw)
 
@@ -141,7 +144,7 @@ class Engine:
     def from_tensors(cls, raw_config: dict, tensors: Dict[str, torch.Tensor], **kw) -> "Engine":
         arch = find_architecture(raw_config)
         cfg = arch.parse(raw_config)
-        spec = arch.spec(cfg, tensors.keys())
+        spec = arch.spec(cfg, {n: tuple(t.shape) for n, t in tensors.items()})
         return cls(spec, DictWeightSource(tensors, tensor_needs(spec), scope=spec.tensor_scope), config=cfg, **kw)
 
     @classmethod

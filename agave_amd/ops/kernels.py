@@ -26,6 +26,7 @@ _SIGNATURES = {
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_gated_act": [_I, _I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
+        "agave_unary_act": [_I, _I, _F, _F, _P, _L, _P, _L, _I, _I, _P],
         "agave_cast": [_I, _P, _I, _P, _L, _P],
         "agave_add_bias": [_I, _P, _L, _P, _I, _I, _P],
         "agave_scale_cap": [_P, _L, _F, _F, _P],
@@ -256,6 +257,25 @@ def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activatio
     n, ff = gate.shape
     library.call(lib("elementwise"), "agave_gated_act", dt(gate), act, ptr(gate), ldg, ptr(up), ldu, ptr(out), ldo, n, ff,
                  stream())
+
+
+# The activations of a feed-forward without a gate: the gate's, and xIELU with two learned numbers.
+UNARY_ACTIVATIONS = dict(GATE_ACTIVATIONS, xielu=4)
+
+
+def unary_act(x: torch.Tensor, out: torch.Tensor, activation: str, p0: float = 0.0, p1: float = 0.0) -> None:
+    """out = act(x), row by row.  ``xielu``: x > 0: p0 x^2 + x/2; x <= 0: p1 (exp(x) - 1 - x) + x/2, where the
+    caller has made p0 = softplus(first learned number) and p1 = 1/2 + softplus(second)."""
+    _dev(x, out)
+    try:
+        act = UNARY_ACTIVATIONS[activation]
+    except KeyError:
+        raise ValueError(f"unary_act: unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}") from None
+    ldx, ldo = _rows(x, "x"), _rows(out, "out")
+    if x.shape != out.shape or x.dtype != out.dtype:
+        raise ValueError("unary_act: x and out must agree in shape and dtype")
+    library.call(lib("elementwise"), "agave_unary_act", dt(x), act, float(p0), float(p1), ptr(x), ldx, ptr(out), ldo,
+                 x.shape[0], x.shape[1], stream())
 
 
 def geglu(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> None:

@@ -1,13 +1,18 @@
 """The parts a layer is put together from, and their registries."""
-from .base import BuildEnv, Workspace, lookup, part_tensors, register, registered
-from . import norm, position, attention, ffn, block  # noqa: F401  (registers the built-in kinds)
+from .base import BuildEnv, Workspace, lookup, mixer_libraries, part_tensors, register, registered, state_tensor
+from . import norm, position, attention, talking_attention, recurrent, parallel, ffn, block  # noqa: F401  (registers the built-in kinds)
 from .attention import Attention
 from .block import PreNormBlock, SandwichBlock, add_pending_and_norm
-from .ffn import GatedFfn
+from .ffn import DenseFfn, GatedFfn
+from .parallel import ParallelMixer
+from .recurrent import GatedDelta, Hgrn2
+from .short_conv import ShortConv
+from .talking_attention import TalkingAttention
 from .linear import Linear
 from .norm import Norm, NormedRows, RmsNorm, add_branch
 from .position import NoPosition, RotaryPosition
 
-__all__ = ["BuildEnv", "Workspace", "lookup", "part_tensors", "register", "registered", "Attention", "GatedFfn",
+__all__ = ["BuildEnv", "Workspace", "lookup", "mixer_libraries", "part_tensors", "register", "registered", "state_tensor",
+           "Attention", "GatedFfn", "DenseFfn", "TalkingAttention", "GatedDelta", "Hgrn2", "ParallelMixer", "ShortConv",
            "Linear", "Norm", "NormedRows", "RmsNorm", "add_branch", "RotaryPosition", "NoPosition", "SandwichBlock", "PreNormBlock",
            "add_pending_and_norm"]

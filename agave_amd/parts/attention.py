@@ -26,7 +26,14 @@ class Attention:
     prompt_steps_can_be_recorded = True        # a multi-token step is the same launches whatever its tokens are
     takes_rows_to_be_normed = True             # its first product may make the normalised rows itself (NormedRows)
 
+    @staticmethod
+    def kernel_libraries(spec, dtype):
+        return ("attention_plain", "attention_mfma") if dtype == torch.bfloat16 else ("attention_plain",)
+
     def __init__(self, spec: AttentionSpec, weights, env: BuildEnv):
+        if getattr(spec.position, "interleaved", False):
+            raise ValueError("attention: the q/k kernel rotates the pairs (i, i + rotary_dim/2); interleaved pairs are "
+                             "the talking attention's")
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
         self.spec = spec

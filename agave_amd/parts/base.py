@@ -147,6 +147,24 @@ def registered(category: str) -> List[str]:
     return sorted(_REGISTRIES[category])
 
 
+def state_tensor(step, memory: int, name: str) -> torch.Tensor:
+    """The fixed-size state ``name`` of a memory: ``[slots, ...]``.  A mixer that stated one
+    :class:`StateNeed` gets that tensor whatever the name; one that stated a dict gets its entry."""
+    held = step.cache.state[memory]
+    return held[name] if isinstance(held, dict) else held
+
+
+def mixer_libraries(spec, dtype) -> set:
+    """The kernel libraries a mixer of this spec runs on (compiled side by side before the model is
+    built).  A class says so with ``kernel_libraries(spec, dtype)``; one that does not is taken to
+    use the attention kernels."""
+    cls = lookup("mixer", spec.kind)
+    own = getattr(cls, "kernel_libraries", None)
+    if own is not None:
+        return set(own(spec, dtype))
+    return {"attention_plain"} | ({"attention_mfma"} if dtype == torch.bfloat16 else set())
+
+
 def part_tensors(obj, _seen=None, _depth=0):
     """Every device tensor a part (and the parts inside it) holds, each once."""
     seen = _seen if _seen is not None else set()

@@ -15,7 +15,9 @@ from typing import List
 
 import torch
 
-from ..config.spec import GatedFfnSpec
+import math
+
+from ..config.spec import DenseFfnSpec, GatedFfnSpec
 from ..ops import kernels
 from ..weights.loader import TensorNeed
 from .base import BuildEnv, register
@@ -67,4 +69,43 @@ class GatedFfn:
         return self.down.forward(act, tag="ffn_down", slices_ok=True)    # the block adds it to the residual stream
 
 
+class DenseFfn:
+    """``W_down act(W_up x)`` without a gate.  The activation is the spec's, one of
+    ``agave_amd.ops.kernels.UNARY_ACTIVATIONS``.  ``xielu`` has two learned numbers p and q in a tensor
+    of its own:  z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2;
+    the two factors are made once at load."""
+    prompt_steps_can_be_recorded = True
+
+    def __init__(self, spec: DenseFfnSpec, weights, env: BuildEnv):
+        if spec.activation not in kernels.UNARY_ACTIVATIONS:
+            raise ValueError(f"dense feed-forward: unsupported activation {spec.activation!r}; "
+                             f"known: {sorted(kernels.UNARY_ACTIVATIONS)}")
+        self.spec, self.env = spec, env
+        self.up = Linear([weights.get(spec.up_proj)], env, "ffn_up")
+        self.down = Linear([weights.get(spec.down_proj)], env, "ffn_down")
+        self.p0 = self.p1 = 0.0
+        if spec.activation == "xielu":
+            if not spec.act_params:
+                raise ValueError("dense feed-forward: xielu needs the tensor of its two numbers")
+            a = weights.get(spec.act_params).to(torch.float64).view(-1)
+            softplus = lambda v: math.log1p(math.exp(-abs(v))) + max(v, 0.0)
+            self.p0, self.p1 = softplus(float(a[0])), 0.5 + softplus(float(a[1]))
+
+    @staticmethod
+    def tensor_needs(spec: DenseFfnSpec) -> List[TensorNeed]:
+        needs = [TensorNeed(spec.up_proj, (spec.intermediate, spec.hidden)),
+                 TensorNeed(spec.down_proj, (spec.hidden, spec.intermediate))]
+        if spec.activation == "xielu":
+            needs.append(TensorNeed(spec.act_params, (2,)))
+        return needs
+
+    def forward(self, x: torch.Tensor, step) -> torch.Tensor:
+        n = x.shape[0]
+        z = self.up.forward(x, tag="ffn_up")
+        act = self.env.workspace.get("ffn_act", n, self.spec.intermediate, z.dtype)
+        kernels.unary_act(z, act, self.spec.activation, self.p0, self.p1)
+        return self.down.forward(act, tag="ffn_down", slices_ok=True)    # the block adds it to the residual stream
+
+
 register("ffn", "gated_dense", GatedFfn)
+register("ffn", "dense", DenseFfn)

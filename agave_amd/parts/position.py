@@ -1,6 +1,6 @@
 """Position encodings applied to queries and keys.
 
-``rope``: rotation of the pairs (i, i + rotary_dim/2) by ``pos/factor * theta^(-2i/rotary_dim)``
+``rope``: rotation of the pairs (i, i + rotary_dim/2), or (2i, 2i + 1) if ``interleaved``, by ``pos/factor * theta^(-2i/rotary_dim)``
 (``src/backend/kernels/cpu/rope.zig:11-48``; linear scaling multiplies the position by
 ``1/factor`` first, ``src/models/gemma3.zig:884-902``).  The frequencies are a table of 32-bit
 floats, rounded once from their exact values; the angle and its sine and cosine are computed
@@ -28,9 +28,20 @@ class RotaryPosition:
         self.inv_freq = torch.from_numpy(inv.astype(np.float32)).to(env.device)
         self.pos_scale = float(np.float32(1.0) / np.float32(spec.factor))
         self.rotary_dim = spec.rotary_dim
+        self.interleaved = bool(spec.interleaved)
+        self._exact = inv / float(spec.factor)
+        self._freq64: Optional[torch.Tensor] = None
+        self._device = env.device
 
     def fused_rotation(self) -> Tuple[Optional[torch.Tensor], float]:
         return self.inv_freq, self.pos_scale
+
+    def rotation_table(self) -> Tuple[Optional[torch.Tensor], bool]:
+        """(frequencies as float64, position scaling folded in; whether the pairs are interleaved), for
+        kernels that make the angle in double."""
+        if self._freq64 is None:
+            self._freq64 = torch.from_numpy(self._exact.astype(np.float64)).to(self._device)
+        return self._freq64, self.interleaved
 
 
 class NoPosition:
@@ -39,6 +50,9 @@ class NoPosition:
 
     def fused_rotation(self) -> Tuple[Optional[torch.Tensor], float]:
         return None, 1.0
+
+    def rotation_table(self) -> Tuple[Optional[torch.Tensor], bool]:
+        return None, False
 
 
 register("position", "rope", RotaryPosition)
