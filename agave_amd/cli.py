@@ -75,8 +75,10 @@ def model_info(engine) -> dict:
             "n_layers": len(s.layers), "max_context": engine.max_context, "dtype": str(engine.dtype).split(".")[-1],
             "bos_token_id": s.bos_token_id, "eos_token_ids": list(s.eos_token_ids),
             "weight_bytes": engine.model.weight_bytes(), "cache_bytes": engine.cache.bytes(),
-            "cache_groups": [{"window": k.window, "n_kv_heads": k.n_kv_heads, "head_dim": k.head_dim}
-                             for k in engine.cache.group_keys]}
+            "cache_groups": [{"window": k.window, "chunk": k.chunk, "n_kv_heads": k.n_kv_heads, "head_dim": k.head_dim,
+                              "v_head_dim": k.v_head_dim or k.head_dim, "layout": k.layout}
+                             for k in engine.cache.group_keys],
+            "state_bytes": sum(t.numel() * t.element_size() for t in engine.cache._state_tensors())}
 
 
 def main(argv: Optional[List[str]] = None) -> int:

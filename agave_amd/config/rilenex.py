@@ -235,4 +235,6 @@ class RilenexConfig:
             architecture=self.architecture, vocab_size=self.vocab, hidden=e, embed_weight="embed", embed_scale=1.0,
             layers=layers, order=[RunEntry(i, i, True) for i in range(len(layers))],
             final_norm=norm("final.norm", e), head_weight="head", max_context=POSITIONS,
-            bos_token_id=None, eos_token_ids=(), tensor_scope=None)
+            bos_token_id=None, eos_token_ids=(),
+            # a tensor that no part asks for (the second norm of a layer without a feed-forward, say) is passed over
+            tensor_scope=())

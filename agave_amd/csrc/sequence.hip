@@ -89,9 +89,9 @@ extern "C" int agave_short_conv(const float* u, long ldu, const float* w, float*
                                 const int* slots, int n_tokens, int n_seqs, int C, int taps, int silu,
                                 int one_token_each, hipStream_t stream) {
     AGAVE_CHECK(n_tokens >= 0 && n_seqs >= 0 && C > 0, "short_conv: bad sizes N=%d B=%d C=%d", n_tokens, n_seqs, C);
-    AGAVE_CHECK(taps >= 2 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (2 to %d are supported)", taps, CONV_MAX_TAPS);
+    AGAVE_CHECK(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps (1 to %d are supported)", taps, CONV_MAX_TAPS);
     AGAVE_CHECK(ldu >= C && ldy >= C, "short_conv: a row stride is below %d", C);
-    AGAVE_CHECK(u && w && y && state && tok_seq && tok_pos && cu && pos0 && slots, "short_conv: null buffer");
+    AGAVE_CHECK(u && w && y && (state || taps == 1) && tok_seq && tok_pos && cu && pos0 && slots, "short_conv: null buffer");
     AGAVE_CHECK(u != y, "short_conv: the convolution is not done in place");
     AGAVE_CHECK(n_tokens < 65536 * 16, "short_conv: too many tokens");
     if (n_tokens == 0) return 0;
@@ -102,7 +102,7 @@ extern "C" int agave_short_conv(const float* u, long ldu, const float* w, float*
     else
         short_conv_kernel<false><<<grid, threads, 0, stream>>>(u, ldu, w, y, ldy, state, tok_seq, tok_pos, pos0, slots, C, taps, one_token_each);
     AGAVE_LAUNCH_CHECK("short_conv");
-    if (!one_token_each) {
+    if (!one_token_each && taps > 1) {
         conv_state_kernel<<<dim3((C + threads - 1) / threads, n_seqs), threads, 0, stream>>>(u, ldu, state, cu, pos0, slots, C, taps);
         AGAVE_LAUNCH_CHECK("conv_state");
     }

@@ -53,8 +53,8 @@ def short_conv(u: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, state: to
     ldu, ldy = _f32rows(u, "conv input", n, c), _f32rows(y, "conv output", n, c)
     if weight.dtype != torch.float32 or not weight.is_contiguous():
         raise TypeError("short_conv: the taps must be a contiguous float32 [channels, taps] tensor")
-    if not 2 <= taps <= MAX_TAPS:
-        raise ValueError(f"short_conv: {taps} taps (2 to {MAX_TAPS} are supported)")
+    if not 1 <= taps <= MAX_TAPS:
+        raise ValueError(f"short_conv: {taps} taps (1 to {MAX_TAPS} are supported)")
     if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (taps - 1, c):
         raise ValueError(f"short_conv: state must be float32 [slots, {taps - 1}, {c}], got {tuple(state.shape)}")
     if max(step.slots) >= state.shape[0]:

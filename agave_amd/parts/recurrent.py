@@ -60,7 +60,7 @@ class GatedDelta:
         self.conv = (ShortConv([weights.get(s.q_conv), weights.get(s.k_conv), weights.get(s.v_conv)], env, silu=True,
                                name="delta_conv") if s.conv_taps else None)
         if self.conv is None:
-            raise ValueError("gated delta rule: the convolution with its SiLU is part of the mixer (conv_taps >= 2)")
+            raise ValueError("gated delta rule: the convolution with its SiLU is part of the mixer (conv_taps >= 1)")
         self.a_log = _vec(weights, s.decay_log, env)
         self.dt_bias = _vec(weights, s.decay_bias, env)
         self.norm_gain = _vec(weights, s.out_norm, env)

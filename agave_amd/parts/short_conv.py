@@ -23,8 +23,8 @@ class ShortConv:
         if len(taps) != 1:
             raise ValueError(f"{name}: stacked convolutions must have the same number of taps, got {sorted(taps)}")
         self.taps = taps.pop()
-        if not 2 <= self.taps <= seq_ops.MAX_TAPS:
-            raise ValueError(f"{name}: {self.taps} taps (2 to {seq_ops.MAX_TAPS} are supported)")
+        if not 1 <= self.taps <= seq_ops.MAX_TAPS:
+            raise ValueError(f"{name}: {self.taps} taps (1 to {seq_ops.MAX_TAPS} are supported)")
         self.weight = torch.cat([w.to(torch.float32) for w in weights], dim=0).contiguous().to(env.device)
         self.channels = self.weight.shape[0]
         self.silu = bool(silu)

@@ -82,19 +82,27 @@ def chunk_talk_attention(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m:
     k = rms_norm(k, W[p + "k.norm"], eps)
     q = rotate_interleaved(q, pos, m["rot"]["dims"], m["rot"]["base"])
     k = rotate_interleaved(k, pos, m["rot"]["dims"], m["rot"]["base"])
-    rep = H // G
-    size = m["mask"]["size"]
     gate = sigmoid(h @ W[p + "g"].T)                                    # [T, H]
+    out = talk_attention_core(q, k, v, W[p + "talk"], m["scale"], m["mask"]["size"]) * gate[:, :, None]
+    return out.reshape(T, H * V) @ W[p + "o"].T
+
+
+def talk_attention_core(q, k, v, talk, scale, chunk, pos0: int = 0):
+    """q [T, H, D], k [T, G, D], v [T, G, V] of positions pos0 .. pos0 + T - 1 (only keys inside this
+    stretch exist).  Scores are mixed across heads by ``talk`` [H, H] (None: not mixed); position i
+    sees j <= i with j // chunk == i // chunk (``chunk`` None: all j <= i).  Returns [T, H, V]."""
+    T, H, _ = q.shape
+    G, V = k.shape[1], v.shape[2]
+    rep = H // G
     out = torch.zeros(T, H, V, dtype=F)
     for t in range(T):
-        lo = (t // size) * size
-        raw = torch.stack([(k[lo:t + 1, hh // rep] @ q[t, hh]) * m["scale"] for hh in range(H)])   # [H, keys]
-        mixed = W[p + "talk"] @ raw
+        lo = 0 if chunk is None else max(0, ((pos0 + t) // chunk) * chunk - pos0)
+        raw = torch.stack([(k[lo:t + 1, hh // rep] @ q[t, hh]) * scale for hh in range(H)])   # [H, keys]
+        mixed = raw if talk is None else talk @ raw
         w = torch.softmax(mixed, dim=-1)
         for hh in range(H):
             out[t, hh] = w[hh] @ v[lo:t + 1, hh // rep]
-    out = out * gate[:, :, None]
-    return out.reshape(T, H * V) @ W[p + "o"].T
+    return out
 
 
 def gated_delta(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, eps: float) -> torch.Tensor:
@@ -111,7 +119,18 @@ def gated_delta(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, ep
     dt = softplus((h @ W[p + "a1"].T) @ W[p + "a2"].T + W[p + "dt_bias"]).view(T, H, D)
     decay = torch.exp(-torch.exp(W[p + "A_log"])[None, :, None] * dt)   # [T, H, D]
     gate = sigmoid((h @ W[p + "g1"].T) @ W[p + "g2"].T).view(T, H, V)
-    S = torch.zeros(H, D, V, dtype=F)
+    o, _ = delta_steps(q, k, v, beta, decay)
+    o = rms(o, eps) * W[p + "norm"] * gate
+    return o.reshape(T, H * V) @ W[p + "o"].T
+
+
+def delta_steps(q, k, v, beta, decay, S=None):
+    """q, k [T, G, D] (already unit vectors), v [T, H, V], beta [T, H], decay [T, H, D]; per head
+    S <- diag(decay) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.  Returns (o [T, H, V], S)."""
+    T, H, V = v.shape
+    G, D = k.shape[1], k.shape[2]
+    rep = H // G
+    S = torch.zeros(H, D, V, dtype=F) if S is None else S.clone()
     o = torch.zeros(T, H, V, dtype=F)
     for t in range(T):
         for hh in range(H):
@@ -120,8 +139,19 @@ def gated_delta(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, ep
             u = beta[t, hh] * (v[t, hh] - S[hh].T @ kk)
             S[hh] = S[hh] + torch.outer(kk, u)
             o[t, hh] = S[hh].T @ qq
-    o = rms(o, eps) * W[p + "norm"] * gate
-    return o.reshape(T, H * V) @ W[p + "o"].T
+    return o, S
+
+
+def forget_steps(q, f, v, S=None):
+    """q, f [T, H, D], v [T, H, V]:  S <- diag(f) S + (1 - f) v^T;  o = S^T q.  Returns (o, S)."""
+    T, H, D = q.shape
+    V = v.shape[2]
+    S = torch.zeros(H, D, V, dtype=F) if S is None else S.clone()
+    o = torch.zeros(T, H, V, dtype=F)
+    for t in range(T):
+        S = f[t][:, :, None] * S + (1.0 - f[t])[:, :, None] * v[t][:, None, :]
+        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    return o, S
 
 
 def parallel_mixer(h, W, p, m, eps):
@@ -138,11 +168,7 @@ def hgrn2(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, eps: flo
     v = (h @ W[p + "v"].T).view(T, H, V)
     low = W[p + "lower"]
     f = (low + (1.0 - low) * sigmoid(h @ W[p + "f"].T + W[p + "f.b"])).view(T, H, D)
-    S = torch.zeros(H, D, V, dtype=F)
-    o = torch.zeros(T, H, V, dtype=F)
-    for t in range(T):
-        S = f[t][:, :, None] * S + (1.0 - f[t])[:, :, None] * v[t][:, None, :]
-        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    o, _ = forget_steps(q, f, v)
     o = rms_norm(o, W[p + "norm"], eps)
     return o.reshape(T, H * V) @ W[p + "o"].T
 
@@ -170,6 +196,73 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
         if layers_out is not None:
             layers_out.append(x.clone())
     return rms_norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+# ---------------------------------------------------------------- random models for the tests
+def random_weights(cfg: dict, seed: int, ranks=(6, 5)) -> Dict[str, torch.Tensor]:
+    """Weights for ``cfg`` as bfloat16-representable float32 tensors, drawn so that every mechanism
+    matters: lower bounds and decays spread over (0, 1), gates away from saturation."""
+    g = torch.Generator().manual_seed(seed)
+    E = cfg["width"]
+
+    def mat(o, i, std=None):
+        return torch.randn(o, i, generator=g) * (std if std is not None else i ** -0.5)
+
+    def vec(n, mean=1.0, std=0.1):
+        return mean + torch.randn(n, generator=g) * std
+
+    W = {"embed": torch.randn(cfg["vocab"], E, generator=g), "final.norm": vec(E), "head": mat(cfg["vocab"], E)}
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", layer["mixer"]
+        W[p + "norm1"] = vec(E)
+        if layer["type"] == "hgrn2":
+            H, D, V = m["heads"], m["dim"], m["vdim"]
+            W.update({p + "mix.q": mat(H * D, E), p + "mix.f": mat(H * D, E), p + "mix.f.b": vec(H * D, 0.0, 0.5),
+                      p + "mix.lower": torch.rand(H * D, generator=g) * 0.9, p + "mix.v": mat(H * V, E),
+                      p + "mix.norm": vec(V), p + "mix.o": mat(E, H * V)})
+        else:
+            l, r = m["left"], m["right"]
+            q = p + "mix.left."
+            H, G, D, V = l["heads"], l["kv_heads"], l["dim"], l["vdim"]
+            W.update({q + "q": mat(H * D, E), q + "k": mat(G * D, E), q + "v": mat(G * V, E),
+                      q + "q.norm": vec(D), q + "k.norm": vec(D),
+                      q + "q.conv": mat(H * D, l["conv"], 0.6), q + "k.conv": mat(G * D, l["conv"], 0.6),
+                      q + "v.conv": mat(G * V, l["conv"], 0.6), q + "talk": torch.eye(H) + mat(H, H, 0.3),
+                      q + "g": mat(H, E), q + "o": mat(E, H * V)})
+            q = p + "mix.right."
+            H, G, D, V = r["heads"], r["kv_heads"], r["dim"], r["vdim"]
+            ra, rg = r.get("decay_rank", ranks[0]), r.get("gate_rank", ranks[1])
+            W.update({q + "q": mat(G * D, E), q + "k": mat(G * D, E), q + "v": mat(H * V, E),
+                      q + "q.conv": mat(G * D, r["conv"], 0.6), q + "k.conv": mat(G * D, r["conv"], 0.6),
+                      q + "v.conv": mat(H * V, r["conv"], 0.6), q + "b": mat(H, E),
+                      q + "A_log": torch.randn(H, generator=g) * 0.5 - 1.0, q + "norm": vec(V),
+                      q + "a1": mat(ra, E), q + "a2": mat(H * D, ra), q + "dt_bias": vec(H * D, -1.0, 1.0),
+                      q + "g1": mat(rg, E), q + "g2": mat(H * V, rg), q + "o": mat(E, H * V)})
+        if layer.get("mlp") is not None:
+            ff = layer["mlp"]["ff"]
+            W.update({p + "norm2": vec(E), p + "mlp.up": mat(ff, E), p + "mlp.down": mat(E, ff),
+                      p + "mlp.act": torch.tensor([0.3, -0.4]) + torch.randn(2, generator=g) * 0.2})
+    return {k: v.bfloat16().float() for k, v in W.items()}
+
+
+def hgrn2_layer(heads, dim, vdim, ff=None):
+    return {"type": "hgrn2", "mixer": {"heads": heads, "dim": dim, "vdim": vdim},
+            "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+
+
+def parallel_layer(left, right, left_scale=0.7, right_scale=1.2, ff=None):
+    """``left``: (heads, kv_heads, dim, vdim, conv, chunk, rot_dims, rot_base); ``right``: (heads, kv_heads, dim, vdim, conv)."""
+    lh, lg, ld, lv, lc, chunk, rot, base = left
+    rh, rg, rd, rv, rc = right
+    return {"type": "parallel", "mlp": None if ff is None else {"kind": "dense", "ff": ff},
+            "mixer": {"left": {"heads": lh, "kv_heads": lg, "dim": ld, "vdim": lv, "conv": lc, "scale": ld ** -0.5,
+                               "mask": {"size": chunk}, "rot": {"dims": rot, "base": base}},
+                      "right": {"heads": rh, "kv_heads": rg, "dim": rd, "vdim": rv, "conv": rc},
+                      "left_scale": left_scale, "right_scale": right_scale}}
+
+
+def config(layers, vocab=131, width=64, eps=1e-5):
+    return {"architecture": "Rilenex", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": list(layers)}
 
 
 def argmax_first(row: torch.Tensor) -> int:
