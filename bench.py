@@ -20,6 +20,14 @@ The other published shapes:
     python bench.py --model 12b --ragged 16 --context 8192        # 16 prompts of unequal lengths 64..4096
     python bench.py --model 27b --prompt-len 2048 --context 8192 --batch 1 --no-points
     python bench.py --model 27b --prompt-len 2048 --context 8192 --batch 32 --no-points
+
+Another design beside the closest Gemma 3 shape of equal size (not the default run):
+
+    python bench.py --design rilenex [--design-size small|medium|large] [--design-layers 8]
+
+prints one JSON line with, for the Rilenex decoder and for a Gemma 3 decoder of the same width, depth,
+heads and about as many weights: tokens a second of a 2,048-token prompt and of decode steps at
+batch 8 and 1, and the time of every kind of kernel in one prompt and in one decode step.
 """
 from __future__ import annotations
 
@@ -190,6 +198,92 @@ def run_prefill(engine, seed: int, repeats: int = 3, length: int = PREFILL_LEN):
     return min(times)
 
 
+# ---------------------------------------------------------------- another design beside Gemma 3
+# width, feed-forward, heads, key heads, head size, chunk of the attention side, inner size of the two-step projections
+DESIGN_SIZES = {"small": (1024, 4096, 8, 2, 128, 128, 64), "medium": (2048, 8192, 16, 4, 128, 256, 128),
+                "large": (4096, 16384, 32, 8, 128, 256, 256)}
+
+
+def rilenex_config(size: str, layers: int) -> dict:
+    """Three layers of HGRN2 to one with attention and the delta rule side by side, every layer with its
+    dense feed-forward; heads of 128 on every side."""
+    e, ff, h, g, d, chunk, rank = DESIGN_SIZES[size]
+    hgrn2 = {"type": "hgrn2", "mixer": {"heads": h, "dim": d, "vdim": d}, "mlp": {"kind": "dense", "ff": ff}}
+    par = {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"left": {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "conv": 4, "scale": d ** -0.5,
+                              "mask": {"size": chunk}, "rot": {"dims": d, "base": 10000.0}},
+                     "right": {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "conv": 4, "decay_rank": rank, "gate_rank": rank},
+                     "left_scale": 1.0, "right_scale": 1.0}}
+    return {"architecture": "Rilenex", "vocab": 32768, "width": e, "norm": {"eps": 1e-5},
+            "layers": [par if i % 4 == 2 else hgrn2 for i in range(layers)]}
+
+
+def gemma_like_config(size: str, layers: int) -> dict:
+    """The same width, depth and heads as a Gemma 3 decoder; its gated feed-forward has three matrices,
+    so two thirds of the inner size give as many weights."""
+    e, ff, h, g, d, chunk, _ = DESIGN_SIZES[size]
+    return dict(GEMMA3_4B, vocab_size=32768, hidden_size=e, num_hidden_layers=layers, num_attention_heads=h,
+                num_key_value_heads=g, head_dim=d, query_pre_attn_scalar=d, intermediate_size=(2 * ff // 3) // 256 * 256,
+                sliding_window=1024, tie_word_embeddings=False)
+
+
+def op_times(engine, prompt_len: int, batch: int, seed: int):
+    """ms of every kind of kernel call in one prompt of ``prompt_len`` tokens and in one decode step
+    of ``batch`` sequences after such prompts (steps run eagerly, two events around each call)."""
+    import torch
+    from agave_amd.engine.generate import RowSampling
+    out = {}
+    prompts = random_prompts(batch, prompt_len, engine.vocab_size, seed)
+    rows = [RowSampling(0.0, 0, 1.0, 1.0, 0.0, []) for _ in range(batch)]
+    slots = [engine.alloc_slot() for _ in range(batch)]
+    engine.enable_profiling(True)
+    try:
+        engine.step_sample(slots[:1], prompts[:1], rows[:1])
+        out["prompt"] = {n: [c, round(ms, 4)] for n, c, ms in engine.profile_table()}
+        toks = [1] * batch
+        if batch > 1:
+            engine.step_sample(slots[1:], prompts[1:], rows[1:])
+        for _ in range(3):
+            toks = engine.step_sample(slots, [[t] for t in toks], rows)
+        from agave_amd.ops import library
+        library.profile.reset()
+        reps = 5
+        for _ in range(reps):
+            toks = engine.step_sample(slots, [[t] for t in toks], rows)
+        out["decode_step"] = {n: [c // reps, round(ms / reps, 4)] for n, c, ms in engine.profile_table()}
+    finally:
+        engine.enable_profiling(False)
+        for s in slots:
+            engine.free_slot(s)
+    return out
+
+
+def compare_designs(args) -> int:
+    import torch
+    from agave_amd.engine import Engine
+    size, layers = args.design_size, args.design_layers
+    context, prompt_len, batch = 4096, 1024, 8
+    result = {"metric": f"{args.design} beside Gemma 3 at equal size ({size}, {layers} layers): tokens/s", "unit": "tokens/s",
+              "dtype": "bf16", "data": "synthetic: uniform-random token ids, random weights", "sizes": DESIGN_SIZES[size],
+              "peaks_measured": measured_peaks()}
+    for name, cfg in ((args.design, rilenex_config(size, layers)), ("gemma3_equal_size", gemma_like_config(size, layers))):
+        engine = Engine.from_random(cfg, seed=0, dtype="bfloat16", max_slots=batch, max_context=context,
+                                    cache_tokens=batch * 2048, device="cuda:0")
+        rec = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
+        pdt = run_prefill(engine, seed=2, length=PREFILL_LEN)
+        rec["prefill_2048"] = {"tokens_per_s": round(PREFILL_LEN / pdt, 1), "ms": round(pdt * 1e3, 3)}
+        for b in (batch, 1):
+            dt, _ = run_decode(engine, b, args.steps, args.warmup, seed=1, prompt_len=prompt_len)
+            rec[f"decode_b{b}"] = {"tokens_per_s": round(b * args.steps / dt, 1), "ms_per_step": round(dt / args.steps * 1e3, 4),
+                                   "weights_gbs": round(engine.model.weight_bytes() / (dt / args.steps) / 1e9, 1)}
+        rec["kernels"] = op_times(engine, PREFILL_LEN, batch, seed=4)
+        result[name] = rec
+        del engine
+        torch.cuda.empty_cache()
+    print(json.dumps(result), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -211,12 +305,19 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
+    ap.add_argument("--design", choices=["rilenex"], help="measure this design beside a Gemma 3 decoder of equal size")
+    ap.add_argument("--design-size", default="medium", choices=sorted(DESIGN_SIZES))
+    ap.add_argument("--design-layers", type=int, default=8)
     args = ap.parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
     if args.gpus != 1 or world != 1:
         if int(os.environ.get("RANK", "0")) == 0:
             print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design:
+        if args.steps == 240:
+            args.steps = 64
+        return compare_designs(args)
     lengths = None
     if args.ragged:
         lengths = ragged_lengths(args.ragged, 64, min(4096, args.context // 2), seed=7)
