@@ -7,7 +7,7 @@
 //   attention over the paged cache with the heads' scores mixed by a matrix before the softmax,
 //     keys of the query's own chunk only (or all earlier keys), a gate per head;
 //   the gated linear recurrence S <- diag(a) S + k u^T, o = S^T q with u = beta (v - S^T k) (delta
-//     rule) or u = v (forget-gate form), the gates made inside;
+//     rule) or u = v (forget-gate form), the gates made inside by waves of their own;
 //   per-head RMS norm of the read-out with an optional elementwise sigmoid gate.
 //
 // Everything between the first product of a mixer and the rows its output product reads is 32-bit
@@ -206,15 +206,15 @@ extern "C" int agave_head_norm_rope_rows(int dtype, const float* q, long ldq, co
 //   w[h][.]    = softmax over the visible keys j: j <= p, and j >= floor(p / chunk) * chunk if chunk > 0
 //   out[h]     = sigmoid(gate[h]) * out_scale * sum_j w[h][j] v_j
 // Keys come in tiles of 64 with a running maximum and sum per head.  Dynamic LDS:
-//   qs[nh*dk] raw[nh*64] mix[nh*64] talk[nh*nh] m[nh] l[nh] alpha[nh] pg[64]
-#define TALK_ACC 16
-template <typename T>
+//   qs[nh*dk] raw[nh*64] mix[nh*64] talk[nh*nh] m[nh] l[nh] alpha[nh] pg[64] vt[64*vcols]
+#define TALK_ACC_MAX 16          // sums a thread: heads x value size up to 256 times this
+template <typename T, int TALK_ACC>
 __global__ __launch_bounds__(256) void talk_attention_kernel(
     const float* __restrict__ q, long ldq, const float* __restrict__ gate, long ldg, T* __restrict__ out, long ldo,
     const T* __restrict__ k_pages, const T* __restrict__ v_pages, const int* __restrict__ table, int width,
     const int* __restrict__ base, int n_pages, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-    const float* __restrict__ talk, int nh, int nkv, int dk, int dv, float scale, int chunk, float out_scale) {
-    extern __shared__ float lds[];
+    const float* __restrict__ talk, int nh, int nkv, int dk, int dv, float scale, int chunk, float out_scale, int vcols) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     float* qs = lds;
     float* raw = qs + (size_t)nh * dk;
     float* mix = raw + (size_t)nh * 64;
@@ -223,6 +223,8 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
     float* l_run = m_run + nh;
     float* alpha = l_run + nh;
     int* pg = reinterpret_cast<int*>(alpha + nh);
+    // [64 keys][vcols], on a 16-byte boundary
+    float* vt = lds + (((size_t)nh * dk + 2 * (size_t)nh * 64 + (size_t)nh * nh + 3 * (size_t)nh + 64 + 3) & ~(size_t)3);
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int t = blockIdx.x;
@@ -238,6 +240,14 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
     float acc[TALK_ACC];
 #pragma unroll
     for (int a = 0; a < TALK_ACC; ++a) acc[a] = 0.f;
+    // which outputs a thread sums: elements tid + 256 a of the token's [nh][dv] row (head and element kept:
+    // no division inside the loops)
+    int one_h[TALK_ACC];                                    // head of accumulator a (nh: none)
+#pragma unroll
+    for (int a = 0; a < TALK_ACC; ++a) {
+        const int idx = tid + a * 256;
+        one_h[a] = idx < nh * dv ? idx / dv : nh;
+    }
     __syncthreads();
 
     for (int j0 = lo; j0 <= p; j0 += 64) {
@@ -253,20 +263,72 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
             pg[tid] = id;
         }
         __syncthreads();
-        // raw scores: lane = key, the waves share the heads
+        // raw scores: lane = key; a wave takes up to four query heads of one key head at a time, so a
+        // key row is read once for them (16 bytes a load where the row's size allows)
         {
             const int j = j0 + lane;
             const int id = pg[lane];
-            for (int h = wv; h < nh; h += 4) {
-                float s = 0.f;
+            const int quads = (rep + 3) / 4, items = nkv * quads;
+            for (int it = wv; it < items; it += 4) {
+                const int g = it / quads, h0 = g * rep + (it % quads) * 4;
+                const int nq = g * rep + rep - h0 < 4 ? g * rep + rep - h0 : 4;
+                const float* q0 = qs + (size_t)h0 * dk;
+                const float* q1 = qs + (size_t)(h0 + (nq > 1 ? 1 : 0)) * dk;
+                const float* q2 = qs + (size_t)(h0 + (nq > 2 ? 2 : 0)) * dk;
+                const float* q3 = qs + (size_t)(h0 + (nq > 3 ? 3 : 0)) * dk;
+                float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
                 if (id >= 0) {
-                    const T* kr = k_pages + (((size_t)id * nkv + h / rep) * AGAVE_PAGE + (j % AGAVE_PAGE)) * dk;
-                    const float* qh = qs + (size_t)h * dk;
-                    float dot = 0.f;
-                    for (int d = 0; d < dk; ++d) dot = fmaf(qh[d], ld(kr + d), dot);
-                    s = dot * scale;
+                    const T* kr = k_pages + (((size_t)id * nkv + g) * AGAVE_PAGE + (j % AGAVE_PAGE)) * dk;
+                    constexpr int VE = 16 / sizeof(T);                  // elements of a 16-byte load
+                    if (dk % VE == 0) {
+                        auto use = [&](const uint4& raw16, int d) {
+                            float kf[VE];
+                            if (sizeof(T) == 2) {
+                                const uint32_t w[4] = {raw16.x, raw16.y, raw16.z, raw16.w};
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) {
+                                    kf[(2 * i) % VE] = __builtin_bit_cast(float, w[i] << 16);
+                                    kf[(2 * i + 1) % VE] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+                                }
+                            } else {
+                                kf[0] = __builtin_bit_cast(float, raw16.x); kf[1] = __builtin_bit_cast(float, raw16.y);
+                                kf[2] = __builtin_bit_cast(float, raw16.z); kf[3] = __builtin_bit_cast(float, raw16.w);
+                            }
+#pragma unroll
+                            for (int i = 0; i < VE; i += 4) {           // dk is a multiple of 4 here: whole float4s of q
+                                const float4 a0 = *reinterpret_cast<const float4*>(q0 + d + i);
+                                const float4 a1 = *reinterpret_cast<const float4*>(q1 + d + i);
+                                const float4 a2 = *reinterpret_cast<const float4*>(q2 + d + i);
+                                const float4 a3 = *reinterpret_cast<const float4*>(q3 + d + i);
+                                d0 = fmaf(a0.x, kf[i], d0); d0 = fmaf(a0.y, kf[i + 1], d0); d0 = fmaf(a0.z, kf[i + 2], d0); d0 = fmaf(a0.w, kf[i + 3], d0);
+                                d1 = fmaf(a1.x, kf[i], d1); d1 = fmaf(a1.y, kf[i + 1], d1); d1 = fmaf(a1.z, kf[i + 2], d1); d1 = fmaf(a1.w, kf[i + 3], d1);
+                                d2 = fmaf(a2.x, kf[i], d2); d2 = fmaf(a2.y, kf[i + 1], d2); d2 = fmaf(a2.z, kf[i + 2], d2); d2 = fmaf(a2.w, kf[i + 3], d2);
+                                d3 = fmaf(a3.x, kf[i], d3); d3 = fmaf(a3.y, kf[i + 1], d3); d3 = fmaf(a3.z, kf[i + 2], d3); d3 = fmaf(a3.w, kf[i + 3], d3);
+                            }
+                        };
+                        const uint4* k16 = reinterpret_cast<const uint4*>(kr);
+                        const int n16 = dk / VE;
+                        int c = 0;
+                        for (; c + 4 <= n16; c += 4) {                  // four loads on their way before the first is used
+                            uint4 b[4];
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) b[i] = k16[c + i];
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) use(b[i], (c + i) * VE);
+                        }
+                        for (; c < n16; ++c) use(k16[c], c * VE);
+                    } else {
+                        for (int d = 0; d < dk; ++d) {
+                            const float kv = ld(kr + d);
+                            d0 = fmaf(q0[d], kv, d0); d1 = fmaf(q1[d], kv, d1);
+                            d2 = fmaf(q2[d], kv, d2); d3 = fmaf(q3[d], kv, d3);
+                        }
+                    }
                 }
-                raw[h * 64 + lane] = s;
+                raw[h0 * 64 + lane] = d0 * scale;
+                if (nq > 1) raw[(h0 + 1) * 64 + lane] = d1 * scale;
+                if (nq > 2) raw[(h0 + 2) * 64 + lane] = d2 * scale;
+                if (nq > 3) raw[(h0 + 3) * 64 + lane] = d3 * scale;
             }
         }
         __syncthreads();
@@ -295,30 +357,71 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
             }
         }
         __syncthreads();
-        // weighted sum of the values: a thread per (head, value element)
+        // weighted sum of the values: a thread per (head, value element); the tile's values of one key
+        // head (up to vcols columns at a time) come into LDS once, in whole rows, and every head of
+        // the group reads them there
 #pragma unroll
         for (int a = 0; a < TALK_ACC; ++a) {
-            const int idx = tid + a * 256;
-            if (idx < nh * dv) {
-                const int h = idx / dv, e = idx % dv;
-                const int kvh = h / rep;
-                float sum = 0.f;
-                for (int r = 0; r < nk; ++r) {
-                    const int id = pg[r];
-                    if (id < 0) continue;
-                    const T* vr = v_pages + (((size_t)id * nkv + kvh) * AGAVE_PAGE + ((j0 + r) % AGAVE_PAGE)) * dv;
-                    sum = fmaf(mix[h * 64 + r], ld(vr + e), sum);
+            if (one_h[a] < nh) acc[a] *= alpha[one_h[a]];
+        }
+        for (int g = 0; g < nkv; ++g) {
+            for (int e0 = 0; e0 < dv; e0 += vcols) {
+                const int ec = dv - e0 < vcols ? dv - e0 : vcols;
+                __syncthreads();                                   // the tile before is read
+                // a wave takes the rows wv, wv + 4, ...; four rows' loads leave before the first is stored
+                // (from clamped addresses, so that none stands under a condition)
+                if (pg[0] >= 0) {
+                    for (int u0 = 0; u0 < 16; u0 += 4) {
+                        if (wv + 4 * u0 >= nk) break;
+                        const T* rowp[4];
+                        bool ok[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int r = wv + 4 * (u0 + u);
+                            ok[u] = r < nk && pg[r] >= 0;
+                            const int rr = ok[u] ? r : 0;
+                            rowp[u] = v_pages + (((size_t)pg[rr] * nkv + g) * AGAVE_PAGE + ((j0 + rr) % AGAVE_PAGE)) * dv + e0;
+                        }
+                        for (int c0 = 0; c0 < ec; c0 += 64) {
+                            const int e = c0 + lane, ee = e < ec ? e : 0;
+                            T got[4];
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) got[u] = rowp[u][ee];
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) {
+                                const int r = wv + 4 * (u0 + u);
+                                if (r < nk && e < ec) vt[r * vcols + e] = ok[u] ? ld(&got[u]) : 0.f;
+                            }
+                        }
+                    }
                 }
-                acc[a] = acc[a] * alpha[h] + sum;
+                __syncthreads();
+                {
+#pragma unroll
+                    for (int a = 0; a < TALK_ACC; ++a) {
+                        const int e = tid + a * 256 - one_h[a] * dv - e0;
+                        if (one_h[a] >= g * rep && one_h[a] < (g + 1) * rep && e >= 0 && e < ec) {
+                            const float* w = mix + one_h[a] * 64;
+                            const float* x = vt + e;
+                            float s0 = 0.f, s1 = 0.f;
+                            int r = 0;
+                            for (; r + 1 < nk; r += 2) {
+                                s0 = fmaf(w[r], x[r * vcols], s0);
+                                s1 = fmaf(w[r + 1], x[(r + 1) * vcols], s1);
+                            }
+                            if (r < nk) s0 = fmaf(w[r], x[r * vcols], s0);
+                            acc[a] += s0 + s1;
+                        }
+                    }
+                }
             }
         }
         __syncthreads();
     }
 #pragma unroll
     for (int a = 0; a < TALK_ACC; ++a) {
-        const int idx = tid + a * 256;
-        if (idx < nh * dv) {
-            const int h = idx / dv;
+        const int h = one_h[a], idx = tid + a * 256;
+        if (h < nh) {
             const float l = l_run[h];
             float o = l > 0.f ? acc[a] / l : 0.f;
             if (gate) o *= sigmoid_f(gate[(size_t)t * ldg + h]);
@@ -334,39 +437,47 @@ extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const f
                                     float out_scale, hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "talk_attention: bad sizes N=%d nh=%d nkv=%d dk=%d dv=%d", N, nh, nkv, dk, dv);
     AGAVE_CHECK(nh % nkv == 0, "talk_attention: %d query heads are not a multiple of %d key heads", nh, nkv);
-    AGAVE_CHECK((long)nh * dv <= 256 * TALK_ACC, "talk_attention: heads x value size %ld exceeds %d", (long)nh * dv, 256 * TALK_ACC);
+    AGAVE_CHECK((long)nh * dv <= 256 * TALK_ACC_MAX, "talk_attention: heads x value size %ld exceeds %d", (long)nh * dv, 256 * TALK_ACC_MAX);
     AGAVE_CHECK(ldq >= (long)nh * dk && ldo >= (long)nh * dv && (!gate || ldg >= nh), "talk_attention: a row stride is too small");
     AGAVE_CHECK(chunk >= 0, "talk_attention: negative chunk");
     AGAVE_CHECK(q && out && k_pages && v_pages && table && base && tok_seq && tok_pos && width > 0 && n_pages > 0,
                 "talk_attention: null buffer or empty table");
-    const size_t lds = ((size_t)nh * dk + 2 * (size_t)nh * 64 + (size_t)nh * nh + 3 * (size_t)nh + 64) * sizeof(float);
+    const size_t fixed = ((size_t)nh * dk + 2 * (size_t)nh * 64 + (size_t)nh * nh + 3 * (size_t)nh + 64 + 4) * sizeof(float);
+    int vcols = 128;                                        // value columns of a key head that are in LDS at a time
+    while (vcols > 16 && (vcols / 2 >= dv || fixed + 64 * vcols * sizeof(float) > 64 * 1024)) vcols /= 2;
+    const size_t lds = fixed + 64 * vcols * sizeof(float);
     AGAVE_CHECK(lds <= 64 * 1024, "talk_attention: %d heads of size %d need %zu bytes of LDS (64 KB are there)", nh, dk, lds);
     if (N == 0) return 0;
-    if (dtype == AGAVE_F32)
-        talk_attention_kernel<float><<<N, 256, lds, stream>>>(q, ldq, gate, ldg, (float*)out, ldo, (const float*)k_pages,
-            (const float*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale);
-    else if (dtype == AGAVE_BF16)
-        talk_attention_kernel<bf16><<<N, 256, lds, stream>>>(q, ldq, gate, ldg, (bf16*)out, ldo, (const bf16*)k_pages,
-            (const bf16*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale);
-    else
+#define TALK_LAUNCH(T, ACC)                                                                                            \
+    talk_attention_kernel<T, ACC><<<N, 256, lds, stream>>>(q, ldq, gate, ldg, (T*)out, ldo, (const T*)k_pages,         \
+        (const T*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale, vcols)
+    const int sums = (nh * dv + 255) / 256;                 // a thread's sums: fewer registers where fewer do
+    if (dtype == AGAVE_F32) {
+        if (sums <= 4) TALK_LAUNCH(float, 4); else if (sums <= 8) TALK_LAUNCH(float, 8); else TALK_LAUNCH(float, 16);
+    } else if (dtype == AGAVE_BF16) {
+        if (sums <= 4) TALK_LAUNCH(bf16, 4); else if (sums <= 8) TALK_LAUNCH(bf16, 8); else TALK_LAUNCH(bf16, 16);
+    } else {
         AGAVE_CHECK(false, "talk_attention: unknown dtype %d", dtype);
+    }
+#undef TALK_LAUNCH
     AGAVE_LAUNCH_CHECK("talk_attention");
     return 0;
 }
 
 // ------------------------------------------------------------------ gated linear recurrence
-// Per sequence and head a state S [dk][dv] of floats, advanced token by token:
+// Per sequence and head a state S [dk][dv] of floats (stored [slot][head][dv][dk]: a column's rows lie
+// together), advanced token by token:
 //     S <- diag(a) S;   u = beta (v - S^T k)  [delta]  or  u = v  [forget gate];   S <- S + k u^T;   o = S^T q
 // so the read-out sees the token's own write.  A column of S (one value element) never meets
-// another, so a workgroup owns 64 columns and four lanes share a column's dk rows (R each).
-// The gates of 16 tokens at a time are made by the whole workgroup into LDS, then the 16 tokens
-// run one after another:
+// another: DS lanes share a column's dk rows (R each), a wave owns 64 / DS columns, and the four
+// consumer waves of a workgroup 4 * 64 / DS columns of one head.  Eight producer waves make the gates
+// of the next TB tokens into the other half of LDS meanwhile (all their loads asked for before the
+// first is used), so that the chain from token to token never waits for memory:
 //   delta:   q, k: unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times dk^-1/2; key head of h is
 //            h / (nh / nkv);  a = exp(-exp(A_log[h]) * softplus(dt[h][d] + dt_bias[h][d]));  beta = sigmoid(b[h])
 //   forget:  q = silu(q);  f = low + (1 - low) sigmoid(f_in + f_bias);  a = f, k = 1 - f
 #define REC_DELTA 0
 #define REC_FORGET 1
-#define REC_TOKENS 16
 
 struct RecurrenceArgs {
     const float* q; long ldq;          // delta: [N, nkv*dk]; forget: [N, nh*dk]
@@ -379,133 +490,222 @@ struct RecurrenceArgs {
     const float* low;                  // forget: [nh*dk]
     const float* f_bias;               // forget: [nh*dk] or null
     float* o; long ldo;                // [N, nh*dv]
-    float* state;                      // [slots][nh][dk][dv]
+    float* state;                      // [slots][nh][dv][dk]
     const int* cu; const int* slots;
     int nh, nkv, dk, dv;
     float unit_eps;                    // delta: inside the root of the unit vectors
 };
 
-__device__ __forceinline__ float quad_sum(float v) {
-    v += dpp_get<0xB1, 0xF>(0.f, v);
-    v += dpp_get<0x4E, 0xF>(0.f, v);
+template <int DS> __device__ __forceinline__ float lanes_sum(float v) {
+    v += dpp_get<0xB1, 0xF>(0.f, v);          // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E, 0xF>(0.f, v);          // quad_perm [2,3,0,1]
+    if (DS == 16) {
+        v += dpp_get<0x141, 0xF>(0.f, v);     // row_half_mirror
+        v += dpp_get<0x140, 0xF>(0.f, v);     // row_mirror
+    }
     return v;
 }
 
-template <int MODE, int R>
-__global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs A) {
-    constexpr int DP = 4 * R;                               // padded rows
-    __shared__ __attribute__((aligned(16))) float sa[REC_TOKENS][DP];
-    __shared__ __attribute__((aligned(16))) float sk[REC_TOKENS][DP];
-    __shared__ __attribute__((aligned(16))) float sq[REC_TOKENS][DP];
-    __shared__ float sv[REC_TOKENS][64];
-    __shared__ float sbeta[REC_TOKENS];
+template <int MODE, int DS, int R, int TB>
+__global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A) {
+    constexpr int DP = DS * R;                              // padded rows
+    constexpr int CW = 64 / DS, CB = 4 * CW;                // columns a wave, a workgroup
+    constexpr int NE = (DP + 63) / 64;                      // elements of a row a producer lane holds
+    constexpr int PW = 8;                                   // producer waves (behind the four consumer waves)
+    constexpr int NT = TB / PW;                             // tokens of a block a producer wave makes
+    __shared__ __attribute__((aligned(16))) float sa[2][TB][DP];
+    __shared__ __attribute__((aligned(16))) float sk[2][TB][DP];
+    __shared__ __attribute__((aligned(16))) float sq[2][TB][DP];
+    __shared__ float sv[2][TB][CB];
+    __shared__ float sbeta[2][TB];
+    __shared__ float skq[2][TB];                            // k . q of a token, for the read-out
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int vl = tid >> 2, ds = tid & 3;
-    const int h = blockIdx.y, s = blockIdx.z;
-    const int col = blockIdx.x * 64 + vl;
+    const bool producer = wv >= 4;
+    const int h = blockIdx.y, s = blockIdx.z, col0 = blockIdx.x * CB;
     const int dk = A.dk, dv = A.dv;
     const int r0 = A.cu[s], r1 = A.cu[s + 1];
-    float* S_g = A.state + (((size_t)A.slots[s] * A.nh + h) * dk) * dv;
+    const int n_blocks = (r1 - r0 + TB - 1) / TB;
 
+    // ---- consumers: their share of the state
+    const int ds = lane & (DS - 1), colb = (wv & 3) * CW + lane / DS, col = col0 + colb;
+    float* S_g = A.state + (((size_t)A.slots[s] * A.nh + h) * dv + (col < dv ? col : 0)) * dk;
     float S[R];
+    if (!producer) {
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-        const int d = ds * R + i;
-        S[i] = (d < dk && col < dv) ? S_g[(size_t)d * dv + col] : 0.f;
+        for (int i = 0; i < R; ++i) {
+            const int d = ds * R + i;
+            S[i] = (d < dk && col < dv) ? S_g[d] : 0.f;
+        }
     }
+    // ---- producers: what does not change from token to token
+    const int pw = wv - 4;
     const int kvh = MODE == REC_DELTA ? h / (A.nh / A.nkv) : h;
+    float c0[NE], c1[NE];                                   // delta: dt_bias, -;  forget: lower bound, the gate's bias
+    float ea = 0.f;
+    if (producer) {
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int d = lane + 64 * e, dd = d < dk ? d : dk - 1;
+            if (MODE == REC_DELTA) { c0[e] = A.dt_bias[(size_t)h * dk + dd]; c1[e] = 0.f; }
+            else { c0[e] = A.low[(size_t)h * dk + dd]; c1[e] = A.f_bias ? A.f_bias[(size_t)h * dk + dd] : 0.f; }
+        }
+        if (MODE == REC_DELTA) ea = expf(A.a_log[h]);
+    }
 
-    for (int tb = r0; tb < r1; tb += REC_TOKENS) {
-        const int nt = r1 - tb < REC_TOKENS ? r1 - tb : REC_TOKENS;
-        __syncthreads();                                    // the tokens before are done with the LDS
-        // ---- the gates of these tokens: a wave per token in turn
-        for (int tt = wv; tt < nt; tt += 4) {
-            const size_t row = (size_t)(tb + tt);
+    // what a producer wave has asked for and not yet used: the rows of its tokens of one block
+    float x0[NT][NE], x1[NT][NE], x2[NT][NE], vv[NT], bb[NT];
+    auto ask = [&](int blk) {
+        const int tb = r0 + blk * TB;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            int row = tb + pw + PW * t;
+            row = row < r1 ? row : r1 - 1;
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                const int d = lane + 64 * e, dd = d < dk ? d : dk - 1;
+                if (MODE == REC_DELTA) {
+                    x0[t][e] = A.q[(size_t)row * A.ldq + (size_t)kvh * dk + dd];
+                    x1[t][e] = A.k[(size_t)row * A.ldk + (size_t)kvh * dk + dd];
+                    x2[t][e] = A.dt[(size_t)row * A.lddt + (size_t)h * dk + dd];
+                } else {
+                    x0[t][e] = A.q[(size_t)row * A.ldq + (size_t)h * dk + dd];
+                    x1[t][e] = A.k[(size_t)row * A.ldk + (size_t)h * dk + dd];
+                    x2[t][e] = 0.f;
+                }
+            }
+            const int c = col0 + (lane < CB ? lane : 0);
+            vv[t] = A.v[(size_t)row * A.ldv + (size_t)h * dv + (c < dv ? c : dv - 1)];
+            bb[t] = MODE == REC_DELTA ? A.b[(size_t)row * A.ldb + h] : 0.f;
+        }
+    };
+    auto make = [&](int blk, int buf) {
+        const int left = r1 - (r0 + blk * TB);              // tokens of this block; the rows behind them leave S as it is
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int tt = pw + PW * t;
+            const bool real = tt < left;
+            float qi = 1.f, ki = 1.f;
             if (MODE == REC_DELTA) {
-                const float* qr = A.q + row * A.ldq + (size_t)kvh * dk;
-                const float* kr = A.k + row * A.ldk + (size_t)kvh * dk;
                 float qq = 0.f, kk = 0.f;
-                for (int d = lane; d < dk; d += 64) { qq = fmaf(qr[d], qr[d], qq); kk = fmaf(kr[d], kr[d], kk); }
+#pragma unroll
+                for (int e = 0; e < NE; ++e)
+                    if (lane + 64 * e < dk) { qq = fmaf(x0[t][e], x0[t][e], qq); kk = fmaf(x1[t][e], x1[t][e], kk); }
                 qq = wave_sum(qq);
                 kk = wave_sum(kk);
-                const float qi = 1.0f / sqrtf(qq + A.unit_eps) / sqrtf((float)dk), ki = 1.0f / sqrtf(kk + A.unit_eps);
-                const float ea = expf(A.a_log[h]);
-                for (int d = lane; d < DP; d += 64) {
-                    float a = 0.f, kx = 0.f, qx = 0.f;
-                    if (d < dk) {
-                        const float x = A.dt[row * A.lddt + (size_t)h * dk + d] + A.dt_bias[(size_t)h * dk + d];
-                        a = expf(-ea * softplus_f(x));
-                        kx = kr[d] * ki;
-                        qx = qr[d] * qi;
-                    }
-                    sa[tt][d] = a; sk[tt][d] = kx; sq[tt][d] = qx;
-                }
-                if (lane == 0) sbeta[tt] = sigmoid_f(A.b[row * A.ldb + h]);
-            } else {
-                for (int d = lane; d < DP; d += 64) {
-                    float a = 0.f, kx = 0.f, qx = 0.f;
-                    if (d < dk) {
-                        const size_t c = (size_t)h * dk + d;
-                        const float lw = A.low[c];
-                        const float f = lw + (1.f - lw) * sigmoid_f(A.k[row * A.ldk + c] + (A.f_bias ? A.f_bias[c] : 0.f));
+                qi = 1.0f / sqrtf(qq + A.unit_eps) / sqrtf((float)dk);
+                ki = 1.0f / sqrtf(kk + A.unit_eps);
+            }
+            float kq = 0.f;
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                const int d = lane + 64 * e;
+                float a = real ? 0.f : 1.f, kx = 0.f, qx = 0.f;
+                if (d < dk && real) {
+                    if (MODE == REC_DELTA) {
+                        a = expf(-ea * softplus_f(x2[t][e] + c0[e]));
+                        kx = x1[t][e] * ki;
+                        qx = x0[t][e] * qi;
+                    } else {
+                        const float f = c0[e] + (1.f - c0[e]) * sigmoid_f(x1[t][e] + c1[e]);
                         a = f;
                         kx = 1.f - f;
-                        qx = silu_f(A.q[row * A.ldq + c]);
+                        qx = silu_f(x0[t][e]);
                     }
-                    sa[tt][d] = a; sk[tt][d] = kx; sq[tt][d] = qx;
                 }
+                kq = fmaf(kx, qx, kq);
+                if (d < DP) { sa[buf][tt][d] = a; sk[buf][tt][d] = kx; sq[buf][tt][d] = qx; }
             }
-            const int c = blockIdx.x * 64 + lane;
-            sv[tt][lane] = c < dv ? A.v[row * A.ldv + (size_t)h * dv + c] : 0.f;
+            kq = wave_sum(kq);
+            if (lane < CB) sv[buf][tt][lane] = real ? vv[t] : 0.f;
+            if (lane == 0) {
+                sbeta[buf][tt] = (MODE == REC_DELTA && real) ? sigmoid_f(bb[t]) : (real ? 1.f : 0.f);
+                skq[buf][tt] = kq;
+            }
         }
-        __syncthreads();
-        // ---- the tokens, one after another
-        for (int tt = 0; tt < nt; ++tt) {
-            const float4* a4 = reinterpret_cast<const float4*>(&sa[tt][ds * R]);
-            const float4* k4 = reinterpret_cast<const float4*>(&sk[tt][ds * R]);
-            const float4* q4 = reinterpret_cast<const float4*>(&sq[tt][ds * R]);
+    };
+
+    // Consumers.  With t = diag(a) S:  S^T k = sum t k,  and the read-out of the new state is
+    // sum t q + u (k . q), so both sums run side by side, one round of cross-lane adds serves both, and
+    // the state's update S = t + k u is all that the next token waits for.  The block's TB tokens are
+    // written out one after another without a branch (rows behind the sequence's end hold a = 1, k = 0).
+    auto consume = [&](int blk, int buf) {
+        const int tb = r0 + blk * TB;
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) {
+            const float4* a4 = reinterpret_cast<const float4*>(&sa[buf][tt][ds * R]);
+            const float4* k4 = reinterpret_cast<const float4*>(&sk[buf][tt][ds * R]);
+            const float4* q4 = reinterpret_cast<const float4*>(&sq[buf][tt][ds * R]);
             float kreg[R];
-            float dot = 0.f;
+            float dk0 = 0.f, dk1 = 0.f, dq0 = 0.f, dq1 = 0.f;
 #pragma unroll
             for (int i = 0; i < R / 4; ++i) {
-                const float4 a = a4[i], k = k4[i];
+                const float4 a = a4[i], k = k4[i], qv = q4[i];
                 kreg[4 * i] = k.x; kreg[4 * i + 1] = k.y; kreg[4 * i + 2] = k.z; kreg[4 * i + 3] = k.w;
                 S[4 * i] *= a.x; S[4 * i + 1] *= a.y; S[4 * i + 2] *= a.z; S[4 * i + 3] *= a.w;
+                dq0 = fmaf(S[4 * i], qv.x, dq0); dq1 = fmaf(S[4 * i + 1], qv.y, dq1);
+                dq0 = fmaf(S[4 * i + 2], qv.z, dq0); dq1 = fmaf(S[4 * i + 3], qv.w, dq1);
                 if (MODE == REC_DELTA) {
-                    dot = fmaf(S[4 * i], k.x, dot); dot = fmaf(S[4 * i + 1], k.y, dot);
-                    dot = fmaf(S[4 * i + 2], k.z, dot); dot = fmaf(S[4 * i + 3], k.w, dot);
+                    dk0 = fmaf(S[4 * i], k.x, dk0); dk1 = fmaf(S[4 * i + 1], k.y, dk1);
+                    dk0 = fmaf(S[4 * i + 2], k.z, dk0); dk1 = fmaf(S[4 * i + 3], k.w, dk1);
                 }
             }
-            float u = sv[tt][vl];
-            if (MODE == REC_DELTA) u = sbeta[tt] * (u - quad_sum(dot));
-            float o = 0.f;
-#pragma unroll
-            for (int i = 0; i < R / 4; ++i) {
-                const float4 qv = q4[i];
-                S[4 * i] = fmaf(kreg[4 * i], u, S[4 * i]); S[4 * i + 1] = fmaf(kreg[4 * i + 1], u, S[4 * i + 1]);
-                S[4 * i + 2] = fmaf(kreg[4 * i + 2], u, S[4 * i + 2]); S[4 * i + 3] = fmaf(kreg[4 * i + 3], u, S[4 * i + 3]);
-                o = fmaf(S[4 * i], qv.x, o); o = fmaf(S[4 * i + 1], qv.y, o);
-                o = fmaf(S[4 * i + 2], qv.z, o); o = fmaf(S[4 * i + 3], qv.w, o);
+            float u = sv[buf][tt][colb];
+            float dq = dq0 + dq1;
+            if (MODE == REC_DELTA) {
+                float dkk = dk0 + dk1;
+                dkk += dpp_get<0xB1, 0xF>(0.f, dkk); dq += dpp_get<0xB1, 0xF>(0.f, dq);
+                dkk += dpp_get<0x4E, 0xF>(0.f, dkk); dq += dpp_get<0x4E, 0xF>(0.f, dq);
+                if (DS == 16) {
+                    dkk += dpp_get<0x141, 0xF>(0.f, dkk); dq += dpp_get<0x141, 0xF>(0.f, dq);
+                    dkk += dpp_get<0x140, 0xF>(0.f, dkk); dq += dpp_get<0x140, 0xF>(0.f, dq);
+                }
+                u = sbeta[buf][tt] * (u - dkk);
+            } else {
+                dq = lanes_sum<DS>(dq);
             }
-            o = quad_sum(o);
-            if (ds == 0 && col < dv) A.o[(size_t)(tb + tt) * A.ldo + (size_t)h * dv + col] = o;
-        }
-    }
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-        const int d = ds * R + i;
-        if (d < dk && col < dv) S_g[(size_t)d * dv + col] = S[i];
+            for (int i = 0; i < R; ++i) S[i] = fmaf(kreg[i], u, S[i]);
+            const float o = fmaf(u, skq[buf][tt], dq);
+            if (ds == 0 && col < dv && tb + tt < r1) A.o[(size_t)(tb + tt) * A.ldo + (size_t)h * dv + col] = o;
+        }
+    };
+
+    // producers run two blocks ahead with their loads and one with their gates
+    if (producer) {
+        ask(0);
+        make(0, 0);
+        if (n_blocks > 1) ask(1);
+    }
+    __syncthreads();
+    for (int blk = 0; blk < n_blocks; ++blk) {
+        if (producer) {
+            if (blk + 1 < n_blocks) {
+                make(blk + 1, (blk + 1) & 1);
+                if (blk + 2 < n_blocks) ask(blk + 2);
+            }
+        } else {
+            consume(blk, blk & 1);
+        }
+        __syncthreads();                                    // the block just read may be overwritten, the one just made be read
+    }
+    if (!producer) {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            const int d = ds * R + i;
+            if (d < dk && col < dv) S_g[d] = S[i];
+        }
     }
 }
 
 template <int MODE>
 static int launch_recurrence(const RecurrenceArgs& A, int n_seqs, hipStream_t stream) {
-    const dim3 grid((A.dv + 63) / 64, A.nh, n_seqs);
-    if (A.dk <= 32) gated_recurrence_kernel<MODE, 8><<<grid, 256, 0, stream>>>(A);
-    else if (A.dk <= 64) gated_recurrence_kernel<MODE, 16><<<grid, 256, 0, stream>>>(A);
-    else if (A.dk <= 128) gated_recurrence_kernel<MODE, 32><<<grid, 256, 0, stream>>>(A);
-    else gated_recurrence_kernel<MODE, 64><<<grid, 256, 0, stream>>>(A);
+    const int cb = A.dk <= 32 ? 64 : 16;                    // columns a workgroup, as the kernel's CB
+    const dim3 grid((A.dv + cb - 1) / cb, A.nh, n_seqs);
+    if (A.dk <= 32) gated_recurrence_kernel<MODE, 4, 8, 16><<<grid, 768, 0, stream>>>(A);
+    else if (A.dk <= 64) gated_recurrence_kernel<MODE, 16, 4, 16><<<grid, 768, 0, stream>>>(A);
+    else if (A.dk <= 128) gated_recurrence_kernel<MODE, 16, 8, 16><<<grid, 768, 0, stream>>>(A);
+    else gated_recurrence_kernel<MODE, 16, 16, 8><<<grid, 768, 0, stream>>>(A);
     AGAVE_LAUNCH_CHECK("gated_recurrence");
     return 0;
 }

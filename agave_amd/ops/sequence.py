@@ -140,7 +140,7 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
                      a_log: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None,
                      lower: Optional[torch.Tensor] = None, f_bias: Optional[torch.Tensor] = None,
                      unit_eps: float = 1e-6) -> None:
-    """Advance ``state`` [slots, heads, dk, dv] over the step's tokens, sequence by sequence, and
+    """Advance ``state`` [slots, heads, dv, dk] (a column of S lies together) over the step's tokens, sequence by sequence, and
     write each token's read-out to ``out`` [N, heads * dv] (float32).
 
     ``DELTA``:  q, k [N, n_kv * dk] become unit vectors per head (q also times dk^-1/2);
@@ -153,8 +153,8 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     kw = (n_kv if mode == DELTA else n_heads) * dk
     ldq, ldk = _f32rows(q, "q", n, kw), _f32rows(k, "k", n, kw)
     ldv, ldo = _f32rows(v, "v", n, n_heads * dv), _f32rows(out, "out", n, n_heads * dv)
-    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, dk, dv):
-        raise ValueError(f"gated_recurrence: state must be float32 [slots, {n_heads}, {dk}, {dv}], got {tuple(state.shape)}")
+    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (n_heads, dv, dk):
+        raise ValueError(f"gated_recurrence: state must be float32 [slots, {n_heads}, {dv}, {dk}], got {tuple(state.shape)}")
     if max(step.slots) >= state.shape[0]:
         raise ValueError("gated_recurrence: a slot lies outside the state")
     lddt = ldb = 0

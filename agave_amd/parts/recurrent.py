@@ -1,6 +1,7 @@
 """Mixers with a matrix of state per head that is advanced token by token.
 
-Both keep ``S`` [head_dim, v_head_dim] per sequence and head in 32-bit and compute, for every token,
+Both keep ``S`` [head_dim, v_head_dim] per sequence and head in 32-bit (stored with a column's rows
+together, ``[heads, v_head_dim, head_dim]``) and compute, for every token,
 
     S <- diag(a) S;   S <- S + k u^T;   o = S^T q          (the read-out sees the token's own write)
 
@@ -86,7 +87,7 @@ class GatedDelta:
 
     def state_need(self) -> Dict[str, StateNeed]:
         s, pre = self.spec, self.state_prefix
-        return {pre + "S": StateNeed((s.n_heads, s.head_dim, s.v_head_dim), torch.float32),
+        return {pre + "S": StateNeed((s.n_heads, s.v_head_dim, s.head_dim), torch.float32),
                 pre + "conv": self.conv.state_need()}
 
     def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0) -> None:
@@ -150,7 +151,7 @@ class Hgrn2:
 
     def state_need(self) -> Dict[str, StateNeed]:
         s = self.spec
-        return {self.state_prefix + "S": StateNeed((s.n_heads, s.head_dim, s.v_head_dim), torch.float32)}
+        return {self.state_prefix + "S": StateNeed((s.n_heads, s.v_head_dim, s.head_dim), torch.float32)}
 
     def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0) -> None:
         s, ws, pre = self.spec, self.env.workspace, self.state_prefix

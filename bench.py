@@ -268,7 +268,7 @@ def compare_designs(args) -> int:
               "peaks_measured": measured_peaks()}
     for name, cfg in ((args.design, rilenex_config(size, layers)), ("gemma3_equal_size", gemma_like_config(size, layers))):
         engine = Engine.from_random(cfg, seed=0, dtype="bfloat16", max_slots=batch, max_context=context,
-                                    cache_tokens=batch * 2048, device="cuda:0")
+                                    cache_tokens=batch * (PREFILL_LEN + 512), device="cuda:0")
         rec = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
         pdt = run_prefill(engine, seed=2, length=PREFILL_LEN)
         rec["prefill_2048"] = {"tokens_per_s": round(PREFILL_LEN / pdt, 1), "ms": round(pdt * 1e3, 3)}

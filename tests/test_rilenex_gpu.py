@@ -93,7 +93,7 @@ def test_state_and_cache_as_the_mixers_asked(models):
     eng = engine(folder, "float32")
     assert set(eng.cache.state) == {0, 1, 2, 3}
     assert set(eng.cache.state[0]) == {"b0.conv", "b1.S", "b1.conv"} and set(eng.cache.state[1]) == {"S"}
-    assert tuple(eng.cache.state[0]["b1.S"].shape[1:]) == (4, 16, 24) and tuple(eng.cache.state[0]["b0.conv"].shape[1:]) == (1, 4 * 24 + 2 * 24 + 2 * 16)
+    assert tuple(eng.cache.state[0]["b1.S"].shape[1:]) == (4, 24, 16) and tuple(eng.cache.state[0]["b0.conv"].shape[1:]) == (1, 4 * 24 + 2 * 24 + 2 * 16)
     keys = eng.cache.group_keys
     assert len(keys) == 2 and {k.chunk for k in keys} == {48, 64} and all(k.layout == "rows" for k in keys)
     assert not eng._prompt_graphs_ok           # mixers with a state run their prompts as they are, never padded

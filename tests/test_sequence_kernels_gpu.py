@@ -274,7 +274,7 @@ def run_recurrence(mode, tensors, sizes, plan_rows, vectors):
     from agave_amd.cache import StateNeed
     from agave_amd.ops import sequence as S
     H, G, dk, dv = sizes
-    cache, planner = planner_for(state={0: StateNeed((H, dk, dv))})
+    cache, planner = planner_for(state={0: StateNeed((H, dv, dk))})
     cache.alloc_slot()
     slot = cache.alloc_slot()
     T = tensors["v"].shape[0]
@@ -285,7 +285,7 @@ def run_recurrence(mode, tensors, sizes, plan_rows, vectors):
         S.gated_recurrence(mode, t["q"], t["k"], t["v"], out[lo:hi], cache.state[0], step, H, G, dk, dv,
                            dt_in=t.get("dt"), beta=t.get("beta"), **{n: x.to(DEV) for n, x in vectors.items()})
         planner.commit(step)
-    return out.cpu().to(F64), cache.state[0][slot].cpu().to(F64)
+    return out.cpu().to(F64), cache.state[0][slot].cpu().to(F64).transpose(1, 2)
 
 
 @pytest.mark.parametrize("H, G, dk, dv", [(4, 2, 16, 24), (3, 3, 20, 12), (2, 1, 64, 64), (2, 2, 100, 70), (1, 1, 130, 8), (5, 1, 8, 3)])
@@ -355,7 +355,7 @@ def test_recurrence_batch_of_unequal_sequences_against_each_alone():
     mk = lambda n: {"q": torch.randn(n, H * dk, generator=g), "k": torch.randn(n, H * dk, generator=g), "v": torch.randn(n, H * dv, generator=g)}
     seqs = [mk(n) for n in lens]
     lower = torch.rand(H * dk, generator=g)
-    cache, planner = planner_for(state={0: StateNeed((H, dk, dv))}, slots=4)
+    cache, planner = planner_for(state={0: StateNeed((H, dv, dk))}, slots=4)
     slots = [cache.alloc_slot() for _ in lens]
     step = feed(cache, planner, slots, lens)
     cat = {n: torch.cat([s[n] for s in seqs]).to(DEV) for n in ("q", "k", "v")}
