@@ -213,7 +213,8 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
     const float* __restrict__ q, long ldq, const float* __restrict__ gate, long ldg, T* __restrict__ out, long ldo,
     const T* __restrict__ k_pages, const T* __restrict__ v_pages, const int* __restrict__ table, int width,
     const int* __restrict__ base, int n_pages, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-    const float* __restrict__ talk, int nh, int nkv, int dk, int dv, float scale, int chunk, float out_scale, int vcols) {
+    const float* __restrict__ talk, int nh, int nkv, int dk, int dv, float scale, int chunk, float out_scale, int vcols,
+    float* __restrict__ parts, int tiles) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* qs = lds;
     float* raw = qs + (size_t)nh * dk;
@@ -250,7 +251,11 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
     }
     __syncthreads();
 
-    for (int j0 = lo; j0 <= p; j0 += 64) {
+    // parts: the launch has a workgroup per tile of 64 keys (blockIdx.y), which leaves its sums, maximum and
+    // weight per head for talk_merge_kernel; a tile behind the query's position leaves none (weight 0)
+    const int j_first = parts ? lo + (int)blockIdx.y * 64 : lo;
+    const int j_last = parts ? (j_first + 63 < p ? j_first + 63 : p) : p;
+    for (int j0 = j_first; j0 <= j_last; j0 += 64) {
         const int nk = p - j0 + 1 < 64 ? p - j0 + 1 : 64;
         if (tid < 64) {
             int id = -1;
@@ -418,6 +423,19 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
         }
         __syncthreads();
     }
+    if (parts) {
+        float* mine = parts + ((size_t)t * tiles + blockIdx.y) * nh * (dv + 2);
+#pragma unroll
+        for (int a = 0; a < TALK_ACC; ++a) {
+            const int h = one_h[a];
+            if (h < nh) mine[(size_t)h * (dv + 2) + (tid + a * 256 - h * dv)] = acc[a];
+        }
+        for (int h = tid; h < nh; h += 256) {
+            mine[(size_t)h * (dv + 2) + dv] = m_run[h];
+            mine[(size_t)h * (dv + 2) + dv + 1] = l_run[h];
+        }
+        return;
+    }
 #pragma unroll
     for (int a = 0; a < TALK_ACC; ++a) {
         const int h = one_h[a], idx = tid + a * 256;
@@ -430,11 +448,33 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
     }
 }
 
+// The tiles' partial results of one (token, head) put together: a wave per pair.
+template <typename T>
+__global__ __launch_bounds__(64) void talk_merge_kernel(const float* __restrict__ parts, int tiles, const float* __restrict__ gate,
+                                                        long ldg, T* __restrict__ out, long ldo, int nh, int dv, float out_scale) {
+    const int t = blockIdx.x / nh, h = blockIdx.x % nh, lane = threadIdx.x;
+    const float* mine = parts + ((size_t)t * tiles * nh + h) * (dv + 2);
+    const size_t step = (size_t)nh * (dv + 2);
+    float m = -INFINITY;
+    for (int i = 0; i < tiles; ++i)
+        if (mine[i * step + dv + 1] > 0.f) m = fmaxf(m, mine[i * step + dv]);
+    float l = 0.f;
+    for (int i = 0; i < tiles; ++i)
+        if (mine[i * step + dv + 1] > 0.f) l += expf(mine[i * step + dv] - m) * mine[i * step + dv + 1];
+    const float g = (gate ? sigmoid_f(gate[(size_t)t * ldg + h]) : 1.f) * out_scale / (l > 0.f ? l : 1.f);
+    for (int e = lane; e < dv; e += 64) {
+        float sum = 0.f;
+        for (int i = 0; i < tiles; ++i)
+            if (mine[i * step + dv + 1] > 0.f) sum = fmaf(expf(mine[i * step + dv] - m), mine[i * step + e], sum);
+        st(out + (size_t)t * ldo + (size_t)h * dv + e, sum * g);
+    }
+}
+
 extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const float* gate, long ldg, void* out, long ldo,
                                     const void* k_pages, const void* v_pages, const int* table, int width,
                                     const int* base, int n_pages, const int* tok_seq, const int* tok_pos,
                                     const float* talk, int N, int nh, int nkv, int dk, int dv, float scale, int chunk,
-                                    float out_scale, hipStream_t stream) {
+                                    float out_scale, float* parts, int tiles, hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "talk_attention: bad sizes N=%d nh=%d nkv=%d dk=%d dv=%d", N, nh, nkv, dk, dv);
     AGAVE_CHECK(nh % nkv == 0, "talk_attention: %d query heads are not a multiple of %d key heads", nh, nkv);
     AGAVE_CHECK((long)nh * dv <= 256 * TALK_ACC_MAX, "talk_attention: heads x value size %ld exceeds %d", (long)nh * dv, 256 * TALK_ACC_MAX);
@@ -449,8 +489,12 @@ extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const f
     AGAVE_CHECK(lds <= 64 * 1024, "talk_attention: %d heads of size %d need %zu bytes of LDS (64 KB are there)", nh, dk, lds);
     if (N == 0) return 0;
 #define TALK_LAUNCH(T, ACC)                                                                                            \
-    talk_attention_kernel<T, ACC><<<N, 256, lds, stream>>>(q, ldq, gate, ldg, (T*)out, ldo, (const T*)k_pages,         \
-        (const T*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale, vcols)
+    talk_attention_kernel<T, ACC><<<grid, 256, lds, stream>>>(q, ldq, gate, ldg, (T*)out, ldo, (const T*)k_pages,      \
+        (const T*)v_pages, table, width, base, n_pages, tok_seq, tok_pos, talk, nh, nkv, dk, dv, scale, chunk, out_scale,  \
+        vcols, parts, tiles)
+    AGAVE_CHECK(!parts || (tiles >= 1 && tiles <= 1024 && chunk > 0 && (long)tiles * 64 >= chunk),
+                "talk_attention: %d tiles of 64 keys do not cover a chunk of %d", tiles, chunk);
+    const dim3 grid(N, parts ? tiles : 1);
     const int sums = (nh * dv + 255) / 256;                 // a thread's sums: fewer registers where fewer do
     if (dtype == AGAVE_F32) {
         if (sums <= 4) TALK_LAUNCH(float, 4); else if (sums <= 8) TALK_LAUNCH(float, 8); else TALK_LAUNCH(float, 16);
@@ -460,6 +504,13 @@ extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const f
         AGAVE_CHECK(false, "talk_attention: unknown dtype %d", dtype);
     }
 #undef TALK_LAUNCH
+    if (parts) {
+        AGAVE_LAUNCH_CHECK("talk_attention");
+        if (dtype == AGAVE_F32)
+            talk_merge_kernel<float><<<N * nh, 64, 0, stream>>>(parts, tiles, gate, ldg, (float*)out, ldo, nh, dv, out_scale);
+        else
+            talk_merge_kernel<bf16><<<N * nh, 64, 0, stream>>>(parts, tiles, gate, ldg, (bf16*)out, ldo, nh, dv, out_scale);
+    }
     AGAVE_LAUNCH_CHECK("talk_attention");
     return 0;
 }
@@ -580,11 +631,12 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
         }
     };
     auto make = [&](int blk, int buf) {
-        const int left = r1 - (r0 + blk * TB);              // tokens of this block; the rows behind them leave S as it is
+        const int left = r1 - (r0 + blk * TB);              // tokens of this block
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const int tt = pw + PW * t;
-            const bool real = tt < left;
+            if (tt >= left) continue;                       // behind the sequence's end: nobody reads that row
+            const bool real = true;
             float qi = 1.f, ki = 1.f;
             if (MODE == REC_DELTA) {
                 float qq = 0.f, kk = 0.f;
@@ -627,47 +679,52 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
 
     // Consumers.  With t = diag(a) S:  S^T k = sum t k,  and the read-out of the new state is
     // sum t q + u (k . q), so both sums run side by side, one round of cross-lane adds serves both, and
-    // the state's update S = t + k u is all that the next token waits for.  The block's TB tokens are
-    // written out one after another without a branch (rows behind the sequence's end hold a = 1, k = 0).
+    // the state's update S = t + k u is all that the next token waits for.
+    auto token = [&](int tb, int buf, int tt) {
+        const float4* a4 = reinterpret_cast<const float4*>(&sa[buf][tt][ds * R]);
+        const float4* k4 = reinterpret_cast<const float4*>(&sk[buf][tt][ds * R]);
+        const float4* q4 = reinterpret_cast<const float4*>(&sq[buf][tt][ds * R]);
+        float kreg[R];
+        float dk0 = 0.f, dk1 = 0.f, dq0 = 0.f, dq1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < R / 4; ++i) {
+            const float4 a = a4[i], k = k4[i], qv = q4[i];
+            kreg[4 * i] = k.x; kreg[4 * i + 1] = k.y; kreg[4 * i + 2] = k.z; kreg[4 * i + 3] = k.w;
+            S[4 * i] *= a.x; S[4 * i + 1] *= a.y; S[4 * i + 2] *= a.z; S[4 * i + 3] *= a.w;
+            dq0 = fmaf(S[4 * i], qv.x, dq0); dq1 = fmaf(S[4 * i + 1], qv.y, dq1);
+            dq0 = fmaf(S[4 * i + 2], qv.z, dq0); dq1 = fmaf(S[4 * i + 3], qv.w, dq1);
+            if (MODE == REC_DELTA) {
+                dk0 = fmaf(S[4 * i], k.x, dk0); dk1 = fmaf(S[4 * i + 1], k.y, dk1);
+                dk0 = fmaf(S[4 * i + 2], k.z, dk0); dk1 = fmaf(S[4 * i + 3], k.w, dk1);
+            }
+        }
+        float u = sv[buf][tt][colb];
+        float dq = dq0 + dq1;
+        if (MODE == REC_DELTA) {
+            float dkk = dk0 + dk1;
+            dkk += dpp_get<0xB1, 0xF>(0.f, dkk); dq += dpp_get<0xB1, 0xF>(0.f, dq);
+            dkk += dpp_get<0x4E, 0xF>(0.f, dkk); dq += dpp_get<0x4E, 0xF>(0.f, dq);
+            if (DS == 16) {
+                dkk += dpp_get<0x141, 0xF>(0.f, dkk); dq += dpp_get<0x141, 0xF>(0.f, dq);
+                dkk += dpp_get<0x140, 0xF>(0.f, dkk); dq += dpp_get<0x140, 0xF>(0.f, dq);
+            }
+            u = sbeta[buf][tt] * (u - dkk);
+        } else {
+            dq = lanes_sum<DS>(dq);
+        }
+#pragma unroll
+        for (int i = 0; i < R; ++i) S[i] = fmaf(kreg[i], u, S[i]);
+        const float o = fmaf(u, skq[buf][tt], dq);
+        if (ds == 0 && col < dv) A.o[(size_t)(tb + tt) * A.ldo + (size_t)h * dv + col] = o;
+    };
     auto consume = [&](int blk, int buf) {
         const int tb = r0 + blk * TB;
+        const int nt = r1 - tb;
+        if (nt >= TB) {                                     // a whole block: its tokens written out one after another
 #pragma unroll
-        for (int tt = 0; tt < TB; ++tt) {
-            const float4* a4 = reinterpret_cast<const float4*>(&sa[buf][tt][ds * R]);
-            const float4* k4 = reinterpret_cast<const float4*>(&sk[buf][tt][ds * R]);
-            const float4* q4 = reinterpret_cast<const float4*>(&sq[buf][tt][ds * R]);
-            float kreg[R];
-            float dk0 = 0.f, dk1 = 0.f, dq0 = 0.f, dq1 = 0.f;
-#pragma unroll
-            for (int i = 0; i < R / 4; ++i) {
-                const float4 a = a4[i], k = k4[i], qv = q4[i];
-                kreg[4 * i] = k.x; kreg[4 * i + 1] = k.y; kreg[4 * i + 2] = k.z; kreg[4 * i + 3] = k.w;
-                S[4 * i] *= a.x; S[4 * i + 1] *= a.y; S[4 * i + 2] *= a.z; S[4 * i + 3] *= a.w;
-                dq0 = fmaf(S[4 * i], qv.x, dq0); dq1 = fmaf(S[4 * i + 1], qv.y, dq1);
-                dq0 = fmaf(S[4 * i + 2], qv.z, dq0); dq1 = fmaf(S[4 * i + 3], qv.w, dq1);
-                if (MODE == REC_DELTA) {
-                    dk0 = fmaf(S[4 * i], k.x, dk0); dk1 = fmaf(S[4 * i + 1], k.y, dk1);
-                    dk0 = fmaf(S[4 * i + 2], k.z, dk0); dk1 = fmaf(S[4 * i + 3], k.w, dk1);
-                }
-            }
-            float u = sv[buf][tt][colb];
-            float dq = dq0 + dq1;
-            if (MODE == REC_DELTA) {
-                float dkk = dk0 + dk1;
-                dkk += dpp_get<0xB1, 0xF>(0.f, dkk); dq += dpp_get<0xB1, 0xF>(0.f, dq);
-                dkk += dpp_get<0x4E, 0xF>(0.f, dkk); dq += dpp_get<0x4E, 0xF>(0.f, dq);
-                if (DS == 16) {
-                    dkk += dpp_get<0x141, 0xF>(0.f, dkk); dq += dpp_get<0x141, 0xF>(0.f, dq);
-                    dkk += dpp_get<0x140, 0xF>(0.f, dkk); dq += dpp_get<0x140, 0xF>(0.f, dq);
-                }
-                u = sbeta[buf][tt] * (u - dkk);
-            } else {
-                dq = lanes_sum<DS>(dq);
-            }
-#pragma unroll
-            for (int i = 0; i < R; ++i) S[i] = fmaf(kreg[i], u, S[i]);
-            const float o = fmaf(u, skq[buf][tt], dq);
-            if (ds == 0 && col < dv && tb + tt < r1) A.o[(size_t)(tb + tt) * A.ldo + (size_t)h * dv + col] = o;
+            for (int tt = 0; tt < TB; ++tt) token(tb, buf, tt);
+        } else {                                            // the sequence's last tokens (a decode step: one)
+            for (int tt = 0; tt < nt; ++tt) token(tb, buf, tt);
         }
     };
 

@@ -22,7 +22,7 @@ kernels.register_signatures(LIBRARY, {
     "agave_head_norm_rope_rows": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _I, _I, _P, _I, _I, _P, _P,
                                   _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "agave_talk_attention": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I,
-                             _F, _I, _F, _P],
+                             _F, _I, _F, _P, _I, _P],
     "agave_gated_recurrence": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _P, _P, _P,
                                _I, _I, _I, _I, _I, _F, _P],
     "agave_head_norm_gate": [_I, _P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _F, _F, _P],
@@ -112,10 +112,14 @@ def check_row_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, dk: 
 
 def talk_attention(q: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor, k_pages: torch.Tensor,
                    v_pages: torch.Tensor, table, base, step, talk: Optional[torch.Tensor], n_heads: int, n_kv: int,
-                   dk: int, dv: int, scale: float, chunk: Optional[int], out_scale: float = 1.0) -> None:
+                   dk: int, dv: int, scale: float, chunk: Optional[int], out_scale: float = 1.0,
+                   parts: Optional[torch.Tensor] = None) -> None:
     """Attention of every token over its sequence's cache rows, the heads' scores mixed by ``talk``
     [heads, heads] before the softmax; keys j <= p of the query's chunk (all if ``chunk`` is None);
-    head h's output times sigmoid(gate[t, h]) (if given) and ``out_scale``, into ``out`` [N, heads * dv]."""
+    head h's output times sigmoid(gate[t, h]) (if given) and ``out_scale``, into ``out`` [N, heads * dv].
+    ``parts`` (float32 [N, tiles, heads, dv + 2], with a chunk only, tiles * 64 >= chunk): a workgroup per
+    token and tile of 64 keys leaves partial results there and a second kernel merges them, which is what
+    a step of few tokens wants (one workgroup per token leaves the chip idle)."""
     _dev(q, gate, out, k_pages, v_pages, table, base, talk)
     n = step.n_tokens
     ldq = _f32rows(q, "q", n, n_heads * dk)
@@ -129,9 +133,16 @@ def talk_attention(q: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Ten
     width = kernels._check_table(table, base, step.tok_seq)
     if chunk is not None and chunk < 1:
         raise ValueError("talk_attention: a chunk holds at least one position")
+    tiles = 0
+    if parts is not None:
+        _dev(parts)
+        if chunk is None or parts.dtype != torch.float32 or not parts.is_contiguous() or parts.dim() != 4 \
+                or tuple(parts.shape[0:1] + parts.shape[2:]) != (n, n_heads, dv + 2) or parts.shape[1] * 64 < chunk:
+            raise ValueError(f"talk_attention: parts must be float32 [{n}, tiles, {n_heads}, {dv + 2}] with tiles * 64 >= chunk")
+        tiles = parts.shape[1]
     library.call(_lib(), "agave_talk_attention", dt(out), ptr(q), ldq, ptr(gate), ldg, ptr(out), ldo, ptr(k_pages),
                  ptr(v_pages), ptr(table), width, ptr(base), n_pages, ptr(step.tok_seq), ptr(step.tok_pos), ptr(talk),
-                 n, n_heads, n_kv, dk, dv, float(scale), int(chunk or 0), float(out_scale), stream())
+                 n, n_heads, n_kv, dk, dv, float(scale), int(chunk or 0), float(out_scale), ptr(parts), tiles, stream())
 
 
 def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,

@@ -26,6 +26,9 @@ from .linear import Linear
 from .short_conv import ShortConv
 
 
+SPLIT_TILES_UP_TO = 64       # steps of up to this many tokens share a token's keys among workgroups
+
+
 class TalkingAttention:
     @staticmethod
     def kernel_libraries(spec, dtype):
@@ -108,8 +111,14 @@ class TalkingAttention:
                                     self.k_norm.gain if self.k_norm else None, self.q_norm.eps if self.q_norm else 0.0,
                                     self.k_norm.eps if self.k_norm else 0.0, self.freq, self.interleaved, step,
                                     k_pages, v_pages, table, base, s.n_heads, s.n_kv_heads, s.head_dim, s.v_head_dim)
+        # few tokens (decode steps): a workgroup per token and tile of 64 keys, merged by a second kernel
+        parts = None
+        if s.chunk is not None and n <= SPLIT_TILES_UP_TO and s.chunk > 64:
+            tiles = (s.chunk + 63) // 64
+            parts = ws.get(pre + "talk_parts", n * tiles, s.n_heads * (s.v_head_dim + 2), torch.float32).view(
+                n, tiles, s.n_heads, s.v_head_dim + 2)
         seq_ops.talk_attention(q_rot, gate, out, k_pages, v_pages, table, base, step, self.talk, s.n_heads, s.n_kv_heads,
-                               s.head_dim, s.v_head_dim, s.scale, s.chunk, scale)
+                               s.head_dim, s.v_head_dim, s.scale, s.chunk, scale, parts=parts)
 
     def forward(self, x: torch.Tensor, step, memory: int, writes: bool = True) -> torch.Tensor:
         ctx = self.env.workspace.get(self.state_prefix + "talk_ctx", x.shape[0], self.context_width, self.env.dtype)

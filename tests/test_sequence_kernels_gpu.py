@@ -159,7 +159,7 @@ def test_head_norm_rotation_and_rows_in_the_cache(interleaved, dk, dv, rot, dtyp
 
 
 # ---------------------------------------------------------------- attention with talking heads
-def run_talk_attention(q, k, v, talk, gate, scale, chunk, dtype, plan, out_scale=1.0):
+def run_talk_attention(q, k, v, talk, gate, scale, chunk, dtype, plan, out_scale=1.0, split=False):
     """Feed one sequence as ``plan`` (row ranges) through the cache; returns [T, H * dv] (float64 on the host)."""
     from agave_amd.cache import GroupKey
     from agave_amd.ops import sequence as S
@@ -178,9 +178,12 @@ def run_talk_attention(q, k, v, talk, gate, scale, chunk, dtype, plan, out_scale
         S.head_norm_rope_rows(q[lo:hi].reshape(hi - lo, -1).float().to(DEV), k[lo:hi].reshape(hi - lo, -1).float().to(DEV),
                               v[lo:hi].reshape(hi - lo, -1).float().to(DEV), q_rows, None, None, 0.0, 0.0, None, False, step,
                               k_pages, v_pages, table, tbase, H, G, dk, dv)
+        parts = None
+        if split and chunk is not None:         # a workgroup per token and tile of 64 keys, then the merge
+            parts = torch.full((hi - lo, (chunk + 63) // 64, H, dv + 2), float("nan"), device=DEV)
         S.talk_attention(q_rows, None if gate is None else gate[lo:hi].float().to(DEV).contiguous(), out[lo:hi], k_pages,
                          v_pages, table, tbase, step, None if talk is None else talk.float().to(DEV), H, G, dk, dv, scale,
-                         chunk, out_scale)
+                         chunk, out_scale, parts=parts)
         planner.commit(step)
     return out.float().cpu().to(F64), cache, slot
 
@@ -201,8 +204,9 @@ def test_talk_attention_prompt_pieces_and_decoding(H, G, dk, dv, chunk, dtype):
     ref = P.talk_attention_core(q.to(F64), k.to(F64), v.to(F64), talk.to(F64), scale, chunk) * P.sigmoid(gate.to(F64))[:, :, None]
     ref = (0.8 * ref).reshape(T, -1)
     tol = 3e-5 if dtype == torch.float32 else 1.5e-2
-    for plan in (cuts(T, T, 1), cuts(T, 130, 1), cuts(T, 3, 2), cuts(T, 50, 47)):
-        got, cache, slot = run_talk_attention(q, k, v, talk, gate, scale, chunk, dtype, plan, out_scale=0.8)
+    for plan, split in ((cuts(T, T, 1), False), (cuts(T, 130, 1), False), (cuts(T, 130, 1), True), (cuts(T, 3, 2), False),
+                        (cuts(T, 50, 47), True)):
+        got, cache, slot = run_talk_attention(q, k, v, talk, gate, scale, chunk, dtype, plan, out_scale=0.8, split=split)
         err = (got - ref).abs().max(-1).values
         assert float(err.max()) <= tol * max(1.0, float(ref.abs().max())), (plan[0], int(err.argmax()), float(err.max()))
         if chunk is not None:                                       # only the pages of the running chunk are still held
@@ -232,7 +236,8 @@ def test_a_key_just_inside_and_just_outside_the_chunk_stands_out(chunk, decode):
         kk[loud, 0, 3] = 30.0
         qq[last, :, 3] = 30.0                                        # score 900 * scale on the loud key
         plan = cuts(T, last, 1) if decode else cuts(T, T, 1)
-        got, _, _ = run_talk_attention(qq, kk, v, None, None, 1.0, chunk, torch.float32, [p for p in plan if p[0] <= last])
+        got, _, _ = run_talk_attention(qq, kk, v, None, None, 1.0, chunk, torch.float32, [p for p in plan if p[0] <= last],
+                                       split=decode)
         ref = P.talk_attention_core(qq.to(F64), kk.to(F64), v.to(F64), None, 1.0, chunk).reshape(T, -1)
         assert torch.allclose(got[last], ref[last], atol=1e-3), (last, loud)
         assert (abs(float(got[last, 0]) - loud) < 1e-3) == seen, (last, loud, float(got[last, 0]))
