@@ -491,17 +491,36 @@ extern "C" int agave_gated_act(int dtype, int act, const void* gate, long ldg, c
 // out = act(x) for a feed-forward without a gate.  Activations 0 to 3 are the gate's; 4 is xIELU with
 // its two factors made by the host:  x > 0: ap x^2 + x/2;  x <= 0: an (exp(x) - 1 - x) + x/2.
 #define AGAVE_UNARY_ACTS 5
+__device__ __forceinline__ float unary_act_value(float z, int act, float p0, float p1) {
+    if (act == 4) return z > 0.f ? fmaf(p0 * z, z, 0.5f * z) : fmaf(p1, expm1f(z) - z, 0.5f * z);
+    return gate_act(z, act);
+}
+
 template <typename T>
 __global__ void unary_act_kernel(const T* __restrict__ x, long ldx, T* __restrict__ out, long ldo, long total, int ff,
                                  int act, float p0, float p1) {
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const long r = idx / ff;
         const int c = (int)(idx % ff);
-        const float z = ld(x + r * ldx + c);
-        float y;
-        if (act == 4) y = z > 0.f ? fmaf(p0 * z, z, 0.5f * z) : fmaf(p1, expm1f(z) - z, 0.5f * z);
-        else y = gate_act(z, act);
-        st(out + r * ldo + c, y);
+        st(out + r * ldo + c, unary_act_value(ld(x + r * ldx + c), act, p0, p1));
+    }
+}
+
+// 16 bytes a thread at a time (rows and strides that are multiples of that): a prompt's rows move at memory's rate
+template <typename T>
+__global__ void unary_act_wide_kernel(const T* __restrict__ x, long ldx, T* __restrict__ out, long ldo, long groups, int per_row,
+                                      int act, float p0, float p1) {
+    constexpr int VE = 16 / sizeof(T);
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < groups; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / per_row;
+        const int c = (int)(idx % per_row) * VE;
+        const uint4 in = *reinterpret_cast<const uint4*>(x + r * ldx + c);
+        const T* v = reinterpret_cast<const T*>(&in);
+        uint4 res;
+        T* o = reinterpret_cast<T*>(&res);
+#pragma unroll
+        for (int i = 0; i < VE; ++i) st(o + i, unary_act_value(ld(v + i), act, p0, p1));
+        *reinterpret_cast<uint4*>(out + r * ldo + c) = res;
     }
 }
 
@@ -514,7 +533,18 @@ extern "C" int agave_unary_act(int dtype, int act, float p0, float p1, const voi
     const long total = (long)n_rows * ff;
     long blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-    if (dtype == AGAVE_F32)
+    const int ve = dtype == AGAVE_F32 ? 4 : 8;
+    const bool wide = (dtype == AGAVE_F32 || dtype == AGAVE_BF16) && ff % ve == 0 && ldx % ve == 0 && ldo % ve == 0 &&
+                      ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0;
+    if (wide) {
+        const long groups = total / ve;
+        long wb = (groups + 255) / 256;
+        if (wb > 65536) wb = 65536;
+        if (dtype == AGAVE_F32)
+            unary_act_wide_kernel<float><<<(int)wb, 256, 0, stream>>>((const float*)x, ldx, (float*)out, ldo, groups, ff / ve, act, p0, p1);
+        else
+            unary_act_wide_kernel<bf16><<<(int)wb, 256, 0, stream>>>((const bf16*)x, ldx, (bf16*)out, ldo, groups, ff / ve, act, p0, p1);
+    } else if (dtype == AGAVE_F32)
         unary_act_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)x, ldx, (float*)out, ldo, total, ff, act, p0, p1);
     else if (dtype == AGAVE_BF16)
         unary_act_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)x, ldx, (bf16*)out, ldo, total, ff, act, p0, p1);

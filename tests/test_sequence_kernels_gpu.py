@@ -391,15 +391,16 @@ def test_head_norm_gate(dtype, H, dv, gated):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_xielu_and_scaled_sum(dtype):
+@pytest.mark.parametrize("cols", [77, 96])            # rows that 16-byte loads do not divide, and rows that they do
+def test_xielu_and_scaled_sum(dtype, cols):
     from agave_amd.ops import kernels, sequence as S
     g = torch.Generator().manual_seed(0)
-    x = (3 * torch.randn(13, 77, generator=g)).to(dtype)
+    x = (3 * torch.randn(13, cols, generator=g)).to(dtype)
     out = torch.empty_like(x, device=DEV)
     p, q = 0.37, -0.61
     kernels.unary_act(x.to(DEV), out, "xielu", math.log1p(math.exp(p)), 0.5 + math.log1p(math.exp(q)))
     tol = 1e-5 if dtype == torch.float32 else 1e-2
     assert torch.allclose(out.float().cpu().to(F64), P.xielu(x.float().to(F64), p, q), atol=tol, rtol=tol)
-    y = torch.randn(13, 77, generator=g).to(dtype)
+    y = torch.randn(13, cols, generator=g).to(dtype)
     S.scaled_sum(x.to(DEV), 0.8, y.to(DEV), 1.1, out)
     assert torch.allclose(out.float().cpu(), 0.8 * x.float() + 1.1 * y.float(), atol=tol * 4, rtol=tol)
