@@ -64,7 +64,7 @@ class TalkSide:
     vdim: int
     conv: int
     scale: float
-    chunk: int
+    chunk: Optional[int]               # None: every earlier key
     rot_dims: int
     rot_base: float
 
@@ -133,8 +133,10 @@ class RilenexConfig:
                 lw, rw = where + ".mixer.left", where + ".mixer.right"
                 l, r = _obj(m, "left", where + ".mixer"), _obj(m, "right", where + ".mixer")
                 rot = _obj(l, "rot", lw)
+                # (a side without a mask sees every earlier key; one without a convolution has none)
+                chunk = _int(_obj(l, "mask", lw), "size", lw + ".mask") if l.get("mask") is not None else None
                 left = TalkSide(_int(l, "heads", lw), _int(l, "kv_heads", lw), _int(l, "dim", lw), _int(l, "vdim", lw),
-                                _int(l, "conv", lw), _num(l, "scale", lw), _int(_obj(l, "mask", lw), "size", lw + ".mask"),
+                                _int(l, "conv", lw, least=0) if l.get("conv") is not None else 0, _num(l, "scale", lw), chunk,
                                 _int(rot, "dims", lw + ".rot", least=0), _num(rot, "base", lw + ".rot", positive=True))
                 right = DeltaSide(_int(r, "heads", rw), _int(r, "kv_heads", rw), _int(r, "dim", rw), _int(r, "vdim", rw),
                                   _int(r, "conv", rw),
@@ -168,7 +170,8 @@ class RilenexConfig:
             else:
                 l, r = m.left, m.right
                 mixer = {"left": {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "conv": l.conv,
-                                  "scale": l.scale, "mask": {"size": l.chunk}, "rot": {"dims": l.rot_dims, "base": l.rot_base}},
+                                  "scale": l.scale, "mask": None if l.chunk is None else {"size": l.chunk},
+                                  "rot": {"dims": l.rot_dims, "base": l.rot_base}},
                          "right": {"heads": r.heads, "kv_heads": r.kv_heads, "dim": r.dim, "vdim": r.vdim, "conv": r.conv},
                          "left_scale": m.left_scale, "right_scale": m.right_scale}
                 for key, val in (("decay_rank", r.decay_rank), ("gate_rank", r.gate_rank)):

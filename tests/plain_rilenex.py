@@ -75,15 +75,16 @@ def chunk_talk_attention(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m:
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     pos = torch.arange(T, dtype=F)
-    q = short_conv(h @ W[p + "q"].T, W[p + "q.conv"]).view(T, H, D)
-    k = short_conv(h @ W[p + "k"].T, W[p + "k.conv"]).view(T, G, D)
-    v = short_conv(h @ W[p + "v"].T, W[p + "v.conv"]).view(T, G, V)
+    q, k, v = h @ W[p + "q"].T, h @ W[p + "k"].T, h @ W[p + "v"].T
+    if p + "q.conv" in W:                                            # a side without a convolution has none
+        q, k, v = short_conv(q, W[p + "q.conv"]), short_conv(k, W[p + "k.conv"]), short_conv(v, W[p + "v.conv"])
+    q, k, v = q.view(T, H, D), k.view(T, G, D), v.view(T, G, V)
     q = rms_norm(q, W[p + "q.norm"], eps)
     k = rms_norm(k, W[p + "k.norm"], eps)
     q = rotate_interleaved(q, pos, m["rot"]["dims"], m["rot"]["base"])
     k = rotate_interleaved(k, pos, m["rot"]["dims"], m["rot"]["base"])
     gate = sigmoid(h @ W[p + "g"].T)                                    # [T, H]
-    out = talk_attention_core(q, k, v, W[p + "talk"], m["scale"], m["mask"]["size"]) * gate[:, :, None]
+    out = talk_attention_core(q, k, v, W[p + "talk"], m["scale"], (m.get("mask") or {}).get("size")) * gate[:, :, None]
     return out.reshape(T, H * V) @ W[p + "o"].T
 
 
@@ -225,10 +226,11 @@ def random_weights(cfg: dict, seed: int, ranks=(6, 5)) -> Dict[str, torch.Tensor
             q = p + "mix.left."
             H, G, D, V = l["heads"], l["kv_heads"], l["dim"], l["vdim"]
             W.update({q + "q": mat(H * D, E), q + "k": mat(G * D, E), q + "v": mat(G * V, E),
-                      q + "q.norm": vec(D), q + "k.norm": vec(D),
-                      q + "q.conv": mat(H * D, l["conv"], 0.6), q + "k.conv": mat(G * D, l["conv"], 0.6),
-                      q + "v.conv": mat(G * V, l["conv"], 0.6), q + "talk": torch.eye(H) + mat(H, H, 0.3),
+                      q + "q.norm": vec(D), q + "k.norm": vec(D), q + "talk": torch.eye(H) + mat(H, H, 0.3),
                       q + "g": mat(H, E), q + "o": mat(E, H * V)})
+            if l.get("conv"):
+                W.update({q + "q.conv": mat(H * D, l["conv"], 0.6), q + "k.conv": mat(G * D, l["conv"], 0.6),
+                          q + "v.conv": mat(G * V, l["conv"], 0.6)})
             q = p + "mix.right."
             H, G, D, V = r["heads"], r["kv_heads"], r["dim"], r["vdim"]
             ra, rg = r.get("decay_rank", ranks[0]), r.get("gate_rank", ranks[1])
@@ -255,8 +257,9 @@ def parallel_layer(left, right, left_scale=0.7, right_scale=1.2, ff=None):
     lh, lg, ld, lv, lc, chunk, rot, base = left
     rh, rg, rd, rv, rc = right
     return {"type": "parallel", "mlp": None if ff is None else {"kind": "dense", "ff": ff},
-            "mixer": {"left": {"heads": lh, "kv_heads": lg, "dim": ld, "vdim": lv, "conv": lc, "scale": ld ** -0.5,
-                               "mask": {"size": chunk}, "rot": {"dims": rot, "base": base}},
+            "mixer": {"left": {"heads": lh, "kv_heads": lg, "dim": ld, "vdim": lv, **({"conv": lc} if lc else {}),
+                               "scale": ld ** -0.5, "mask": None if chunk is None else {"size": chunk},
+                               "rot": {"dims": rot, "base": base}},
                       "right": {"heads": rh, "kv_heads": rg, "dim": rd, "vdim": rv, "conv": rc},
                       "left_scale": left_scale, "right_scale": right_scale}}
 

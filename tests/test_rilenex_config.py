@@ -63,12 +63,27 @@ def test_inner_sizes_come_from_the_checkpoint():
     assert "l1.mix.lower" in str(e.value) and "l0.mix.left.talk" in str(e.value)
 
 
+def test_a_side_without_mask_or_convolution():
+    raw = copy.deepcopy(small_config())
+    left = raw["layers"][0]["mixer"]["left"]
+    left["mask"] = None
+    left.pop("conv")
+    cfg = RilenexConfig.from_dict(raw)
+    assert cfg.layers[0].mixer.left.chunk is None and cfg.layers[0].mixer.left.conv == 0
+    spec = cfg.model_spec(None)
+    talk = spec.layers[0].mixer.branches[0]
+    assert talk.chunk is None and talk.conv_taps == 0
+    assert not any(n.name.endswith("left.q.conv") for n in tensor_needs(spec))
+    assert RilenexConfig.from_dict(cfg.to_dict()) == cfg
+
+
 @pytest.mark.parametrize("edit, word", [
     (lambda c: c.pop("vocab"), "vocab"),
     (lambda c: c["layers"][0].__setitem__("type", "other"), "unknown layer type"),
     (lambda c: c["layers"][0]["mixer"]["left"].__setitem__("kv_heads", 3), "multiple"),
     (lambda c: c["layers"][0]["mixer"]["left"]["rot"].__setitem__("dims", 26), "rot"),
     (lambda c: c["layers"][0]["mixer"]["left"]["mask"].pop("size"), "size"),
+    (lambda c: c["layers"][0]["mixer"]["right"].pop("conv"), "conv"),
     (lambda c: c["layers"][2].__setitem__("mlp", {"kind": "routed", "ff": 8}), "dense"),
     (lambda c: c["norm"].__setitem__("eps", 0), "eps"),
 ])

@@ -26,6 +26,8 @@ CONFIGS = {
     # a width that is no multiple of 8 (no matrix-core packing), one key head, a chunk longer than a page, taps of 1
     "odd": lambda: P.config([P.hgrn2_layer(5, 12, 28, ff=50),
                              P.parallel_layer((6, 1, 20, 10, 1, 100, 8, 77.0), (3, 1, 24, 20, 4), ff=None)], vocab=97, width=60),
+    # the attention side without a mask (every earlier key) and without a convolution, no rotation, heads of 18
+    "no_mask": lambda: P.config([P.parallel_layer((3, 3, 18, 14, 0, None, 0, 10.0), (2, 1, 12, 18, 3), ff=44)], vocab=89, width=48),
     "hgrn2_alone": lambda: P.config([P.hgrn2_layer(6, 40, 24)], vocab=101, width=72),
     "parallel_alone": lambda: P.config([P.parallel_layer((8, 4, 32, 32, 3, 32, 32, 250.0), (4, 4, 32, 48, 4))], vocab=101, width=72),
 }

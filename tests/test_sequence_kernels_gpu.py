@@ -189,7 +189,7 @@ def run_talk_attention(q, k, v, talk, gate, scale, chunk, dtype, plan, out_scale
 
 
 @pytest.mark.parametrize("H, G, dk, dv, chunk", [(4, 2, 24, 16, 48), (3, 3, 40, 40, 64), (6, 1, 16, 20, 100), (2, 1, 72, 8, None),
-                                                 (5, 5, 8, 130, 7)])
+                                                 (5, 5, 8, 130, 7), (9, 3, 18, 6, 200)])      # (18: no 16-byte loads of a key row)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_talk_attention_prompt_pieces_and_decoding(H, G, dk, dv, chunk, dtype):
     T = 215
