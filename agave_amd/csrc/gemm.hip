@@ -1,6 +1,8 @@
 // Plain tiled matrix product for gfx950: C[M,N] = A[M,K] * W[N,K]^T with 32-bit
 // accumulation, for any M, N, K and any mix of float / bf16 operands.
 //
+// (a kernel of its own takes up to 16 rows of A: decode steps).
+//
 // This is the true 32-bit path of the linear layers (ordinary fused multiply-adds, no
 // reduced-precision matrix mode) and the fallback for sizes the MFMA kernels refuse.
 // Weights are row-major [out, in] and used as y = W x, as in the reference
@@ -63,9 +65,42 @@ __global__ __launch_bounds__(256) void gemm_tn_kernel(const TA* __restrict__ A, 
     }
 }
 
+// Up to FEW_ROWS rows of A (a decode step's tokens): a wave per column of C, the lanes along K, so a
+// weight row is read once, in whole lines, and the few rows of A come from the cache; the tiled kernel
+// above would fill a sixteenth of its tile and wait at two barriers per 16 columns of K.
+#define FEW_ROWS 16
+template <typename TA, typename TW, typename TC>
+__global__ __launch_bounds__(256) void gemm_few_rows_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W,
+                                                            long ldw, TC* __restrict__ C, long ldc, int M, int N, int K) {
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const TW* w = W + (size_t)n * ldw;
+    float acc[FEW_ROWS];
+#pragma unroll
+    for (int m = 0; m < FEW_ROWS; ++m) acc[m] = 0.f;
+    for (int k = lane; k < K; k += 64) {
+        const float wk = ld(w + k);
+#pragma unroll
+        for (int m = 0; m < FEW_ROWS; ++m)
+            if (m < M) acc[m] = fmaf(ld(A + (size_t)m * lda + k), wk, acc[m]);
+    }
+#pragma unroll
+    for (int m = 0; m < FEW_ROWS; ++m) {
+        if (m < M) {                                        // (M is the same for every lane)
+            const float sum = wave_sum(acc[m]);
+            if (lane == 0) st(C + (size_t)m * ldc + n, sum);
+        }
+    }
+}
+
 template <typename TA, typename TW, typename TC>
 static void launch_gemm(const void* A, long lda, const void* W, long ldw, void* C, long ldc, int M, int N, int K,
                         hipStream_t stream) {
+    if (M <= FEW_ROWS) {
+        gemm_few_rows_kernel<TA, TW, TC><<<(N + 3) / 4, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, ldw, (TC*)C, ldc, M, N, K);
+        return;
+    }
     dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
     gemm_tn_kernel<TA, TW, TC><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, ldw, (TC*)C, ldc, M, N, K);
 }
