@@ -2,10 +2,12 @@
 ``scales[i] * branch_i(x)``.
 
 Branches that can hand over the rows their output product reads (``context_into`` with
-``context_width`` and ``o_weight``: the built-in mixers with a state do) write them, already times
-their scale, side by side into one buffer, and one product with the branches' output matrices put
-next to each other along the columns makes the weighted sum: ``[W_1 W_2] [s_1 c_1; s_2 c_2]``.  Any
-other pair of branches runs its own ``forward`` and a small kernel adds the two results.
+``context_width``, ``o_weight`` and ``input_matrices``: the built-in mixers with a state do) share
+their first product too (all their matrices stacked, one launch, the 32-bit rows shared out by
+columns) and write their rows, already times their scale, side by side into one buffer; one product
+with the branches' output matrices put next to each other along the columns makes the weighted
+sum: ``[W_1 W_2] [s_1 c_1; s_2 c_2]``.  Any other pair of branches runs its own ``forward`` and a
+small kernel adds the two results.
 
 At most one branch may keep keys and values in the cache (a memory has one group of pages); every
 branch's fixed-size state lives in the memory under the branch's own prefix (``b0.``, ``b1.``, ...).
@@ -35,13 +37,21 @@ class ParallelMixer:
             raise ValueError("branches that do not hand over their output product's rows are summed in pairs only")
         self.branches = []
         for i, (b, c) in enumerate(zip(spec.branches, classes)):
-            part = c(b, weights, env, own_output=False) if self.fused else c(b, weights, env)
+            part = c(b, weights, env, own_output=False, own_input=False) if self.fused else c(b, weights, env)
             part.state_prefix = f"b{i}."
             self.branches.append(part)
         if sum(1 for p in self.branches if p.kv_need() is not None) > 1:
             raise ValueError("a parallel mixer: at most one branch may keep keys and values in the cache")
-        self.o = None
+        self.o = self.inp = None
         if self.fused:
+            # every branch reads the same rows: their first products are one, its 32-bit rows shared out by columns
+            firsts = [m for p in self.branches for m in p.input_matrices]
+            for p in self.branches:
+                p.input_matrices = None
+            self.inp = Linear(firsts, env, "parallel_in")
+            self.in_bounds = [0]
+            for p in self.branches:
+                self.in_bounds.append(self.in_bounds[-1] + p.input_width)
             mats = [p.o_weight for p in self.branches]
             for p in self.branches:
                 p.o_weight = None
@@ -89,8 +99,10 @@ class ParallelMixer:
         ws, n = self.env.workspace, x.shape[0]
         if self.fused:
             ctx = ws.get("parallel_ctx", n, self.bounds[-1], self.env.dtype)
-            for p, view, scale in zip(self.branches, ws.columns(ctx, tuple(self.bounds)), self.spec.scales):
-                p.context_into(x, step, memory, writes, view, scale)
+            first = self.inp.forward(x, out_dtype=torch.float32, tag="parallel_in")
+            for p, view, rows, scale in zip(self.branches, ws.columns(ctx, tuple(self.bounds)),
+                                            ws.columns(first, tuple(self.in_bounds)), self.spec.scales):
+                p.context_into(x, step, memory, writes, view, scale, proj=rows)
             return self.o.forward(ctx, tag="parallel_o", slices_ok=True)
         a = self.branches[0].forward(x, step, memory, writes)
         b = self.branches[1].forward(x, step, memory, writes)

@@ -42,7 +42,7 @@ class GatedDelta:
     def kernel_libraries(spec, dtype):
         return ("sequence",)
 
-    def __init__(self, spec: GatedDeltaSpec, weights, env: BuildEnv, own_output: bool = True):
+    def __init__(self, spec: GatedDeltaSpec, weights, env: BuildEnv, own_output: bool = True, own_input: bool = True):
         s = spec
         if s.n_heads % s.n_kv_heads:
             raise ValueError("heads must be a multiple of the query/key heads")
@@ -52,8 +52,10 @@ class GatedDelta:
         self.context_width = self.vd
         a1, g1 = weights.get(s.decay_in), weights.get(s.gate_in)
         # q, k, v, the write strength's logit and the inner rows of the decay and of the gate: one product
-        self.proj = Linear([weights.get(s.q_proj), weights.get(s.k_proj), weights.get(s.v_proj), weights.get(s.beta_proj),
-                            a1, g1], env, "delta_in")
+        mats = [weights.get(s.q_proj), weights.get(s.k_proj), weights.get(s.v_proj), weights.get(s.beta_proj), a1, g1]
+        self.input_matrices = None if own_input else mats
+        self.input_width = sum(int(m.shape[0]) for m in mats)
+        self.proj = Linear(mats, env, "delta_in") if own_input else None
         self.ra, self.rg = int(a1.shape[0]), int(g1.shape[0])
         # the second steps read 32-bit rows, so they run on the plain product whatever the engine's type
         self.decay_out = Linear([weights.get(s.decay_out)], env, "delta_decay", pack=False)
@@ -90,12 +92,14 @@ class GatedDelta:
         return {pre + "S": StateNeed((s.n_heads, s.v_head_dim, s.head_dim), torch.float32),
                 pre + "conv": self.conv.state_need()}
 
-    def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0) -> None:
+    def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0,
+                     proj: Optional[torch.Tensor] = None) -> None:
         s, ws, pre = self.spec, self.env.workspace, self.state_prefix
         n = x.shape[0]
         if not writes:
             raise ValueError("a recurrent mixer advances its own state; it cannot read another run's")
-        proj = self.proj.forward(x, out_dtype=torch.float32, tag=pre + "delta_in")
+        if proj is None:
+            proj = self.proj.forward(x, out_dtype=torch.float32, tag=pre + "delta_in")
         c_qkv = 2 * self.kd + self.vd
         bounds = (0, c_qkv, c_qkv + s.n_heads, c_qkv + s.n_heads + self.ra, c_qkv + s.n_heads + self.ra + self.rg)
         qkv, beta, a_in, g_in = ws.columns(proj, bounds)
@@ -121,13 +125,16 @@ class Hgrn2:
     def kernel_libraries(spec, dtype):
         return ("sequence",)
 
-    def __init__(self, spec: Hgrn2Spec, weights, env: BuildEnv, own_output: bool = True):
+    def __init__(self, spec: Hgrn2Spec, weights, env: BuildEnv, own_output: bool = True, own_input: bool = True):
         s = spec
         self.spec, self.env = spec, env
         self.state_prefix = ""
         self.hd, self.vd = s.n_heads * s.head_dim, s.n_heads * s.v_head_dim
         self.context_width = self.vd
-        self.proj = Linear([weights.get(s.q_proj), weights.get(s.f_proj), weights.get(s.v_proj)], env, "hgrn2_in")
+        mats = [weights.get(s.q_proj), weights.get(s.f_proj), weights.get(s.v_proj)]
+        self.input_matrices = None if own_input else mats
+        self.input_width = sum(int(m.shape[0]) for m in mats)
+        self.proj = Linear(mats, env, "hgrn2_in") if own_input else None
         self.f_bias = _vec(weights, s.f_bias, env) if s.f_bias else None      # added inside the recurrence's kernel
         self.lower = _vec(weights, s.lower, env)
         self.norm_gain = _vec(weights, s.out_norm, env)
@@ -153,12 +160,14 @@ class Hgrn2:
         s = self.spec
         return {self.state_prefix + "S": StateNeed((s.n_heads, s.v_head_dim, s.head_dim), torch.float32)}
 
-    def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0) -> None:
+    def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0,
+                     proj: Optional[torch.Tensor] = None) -> None:
         s, ws, pre = self.spec, self.env.workspace, self.state_prefix
         n = x.shape[0]
         if not writes:
             raise ValueError("a recurrent mixer advances its own state; it cannot read another run's")
-        proj = self.proj.forward(x, out_dtype=torch.float32, tag=pre + "hgrn2_in")
+        if proj is None:
+            proj = self.proj.forward(x, out_dtype=torch.float32, tag=pre + "hgrn2_in")
         q, f, v = ws.columns(proj, (0, self.hd, 2 * self.hd, 2 * self.hd + self.vd))
         o = ws.get(pre + "hgrn2_readout", n, self.vd, torch.float32)
         seq_ops.gated_recurrence(seq_ops.FORGET, q, f, v, o, state_tensor(step, memory, pre + "S"), step, s.n_heads,

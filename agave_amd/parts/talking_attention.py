@@ -34,7 +34,7 @@ class TalkingAttention:
     def kernel_libraries(spec, dtype):
         return ("sequence",)
 
-    def __init__(self, spec: TalkingAttentionSpec, weights, env: BuildEnv, own_output: bool = True):
+    def __init__(self, spec: TalkingAttentionSpec, weights, env: BuildEnv, own_output: bool = True, own_input: bool = True):
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")
         self.spec, self.env = spec, env
@@ -45,7 +45,10 @@ class TalkingAttention:
         mats = [weights.get(s.q_proj), weights.get(s.k_proj), weights.get(s.v_proj)]
         if s.gate_proj:
             mats.append(weights.get(s.gate_proj))
-        self.proj = Linear(mats, env, "talk_qkvg")
+        # (side by side with other mixers, the first products of all of them are one: the parent takes the matrices)
+        self.input_matrices = None if own_input else mats
+        self.input_width = sum(int(m.shape[0]) for m in mats)
+        self.proj = Linear(mats, env, "talk_qkvg") if own_input else None
         self.conv = (ShortConv([weights.get(s.q_conv), weights.get(s.k_conv), weights.get(s.v_conv)], env, silu=False,
                                name="talk_conv") if s.conv_taps else None)
         self.q_norm = lookup("norm", s.q_norm.kind)(s.q_norm, weights, env) if s.q_norm else None
@@ -89,15 +92,18 @@ class TalkingAttention:
     def state_need(self) -> Optional[Dict[str, StateNeed]]:
         return {self.state_prefix + "conv": self.conv.state_need()} if self.conv is not None else None
 
-    def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0) -> None:
-        """The rows that the output product reads, times ``scale``, into ``out`` [N, context_width]."""
+    def context_into(self, x: torch.Tensor, step, memory: int, writes: bool, out: torch.Tensor, scale: float = 1.0,
+                     proj: Optional[torch.Tensor] = None) -> None:
+        """The rows that the output product reads, times ``scale``, into ``out`` [N, context_width].
+        ``proj``: the first product's 32-bit rows [N, input_width], if the caller made them."""
         s, ws, pre = self.spec, self.env.workspace, self.state_prefix
         n = x.shape[0]
         if not writes:
             raise ValueError("talking attention keeps a convolution state and a cache of its own; it cannot read another run's")
         k_pages, v_pages, _ = step.cache.pages_of(memory)
         table, base = step.tables[step.cache.group_of_memory[memory]]
-        proj = self.proj.forward(x, out_dtype=torch.float32, tag=pre + "talk_qkvg")
+        if proj is None:
+            proj = self.proj.forward(x, out_dtype=torch.float32, tag=pre + "talk_qkvg")
         lo = self.qd + self.kd + self.vd
         qkv = proj[:, :lo]
         gate = proj[:, lo:lo + s.n_heads] if s.gate_proj else None
