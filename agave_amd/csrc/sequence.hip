@@ -547,6 +547,34 @@ struct RecurrenceArgs {
     float unit_eps;                    // delta: inside the root of the unit vectors
 };
 
+// A lane's R rows of its state column, to and from memory: 16 bytes at a time where the column's
+// length allows (R is a multiple of 4, so a lane's rows start at a multiple of 4 too).
+template <int R> __device__ __forceinline__ void state_load(float (&S)[R], const float* col_ptr, int d0, int dk, bool live) {
+    if ((dk & 3) == 0) {
+#pragma unroll
+        for (int i = 0; i < R; i += 4) {
+            float4 x = {0.f, 0.f, 0.f, 0.f};
+            if (live && d0 + i < dk) x = *reinterpret_cast<const float4*>(col_ptr + d0 + i);
+            S[i] = x.x; S[i + 1] = x.y; S[i + 2] = x.z; S[i + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i) S[i] = (live && d0 + i < dk) ? col_ptr[d0 + i] : 0.f;
+    }
+}
+template <int R> __device__ __forceinline__ void state_store(const float (&S)[R], float* col_ptr, int d0, int dk, bool live) {
+    if (!live) return;
+    if ((dk & 3) == 0) {
+#pragma unroll
+        for (int i = 0; i < R; i += 4)
+            if (d0 + i < dk) *reinterpret_cast<float4*>(col_ptr + d0 + i) = float4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+    } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+            if (d0 + i < dk) col_ptr[d0 + i] = S[i];
+    }
+}
+
 template <int DS> __device__ __forceinline__ float lanes_sum(float v) {
     v += dpp_get<0xB1, 0xF>(0.f, v);          // quad_perm [1,0,3,2]
     v += dpp_get<0x4E, 0xF>(0.f, v);          // quad_perm [2,3,0,1]
@@ -582,13 +610,7 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
     const int ds = lane & (DS - 1), colb = (wv & 3) * CW + lane / DS, col = col0 + colb;
     float* S_g = A.state + (((size_t)A.slots[s] * A.nh + h) * dv + (col < dv ? col : 0)) * dk;
     float S[R];
-    if (!producer) {
-#pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int d = ds * R + i;
-            S[i] = (d < dk && col < dv) ? S_g[d] : 0.f;
-        }
-    }
+    if (!producer) state_load<R>(S, S_g, ds * R, dk, col < dv);
     // ---- producers: what does not change from token to token
     const int pw = wv - 4;
     const int kvh = MODE == REC_DELTA ? h / (A.nh / A.nkv) : h;
@@ -746,13 +768,112 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
         }
         __syncthreads();                                    // the block just read may be overwritten, the one just made be read
     }
-    if (!producer) {
+    if (!producer) state_store<R>(S, S_g, ds * R, dk, col < dv);
+}
+
+// One token per sequence (a decode step): four waves, each with 64 / DS columns, and every wave makes
+// the token's gates for itself, so nothing waits for another wave's work and a compute unit holds eight
+// such workgroups (the kernel above, with its twelve waves, holds one: 1,024 workgroups took four rounds).
+template <int MODE, int DS, int R>
+__global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceArgs A) {
+    constexpr int DP = DS * R, CW = 64 / DS, CB = 4 * CW, NE = (DP + 63) / 64;
+    __shared__ __attribute__((aligned(16))) float sa[4][DP];
+    __shared__ __attribute__((aligned(16))) float sk[4][DP];
+    __shared__ __attribute__((aligned(16))) float sq[4][DP];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int h = blockIdx.y, s = blockIdx.z, col0 = blockIdx.x * CB;
+    const int dk = A.dk, dv = A.dv;
+    const size_t row = (size_t)A.cu[s];
+    const int ds = lane & (DS - 1), col = col0 + wv * CW + lane / DS;
+    float* S_g = A.state + (((size_t)A.slots[s] * A.nh + h) * dv + (col < dv ? col : 0)) * dk;
+    float S[R];
+    state_load<R>(S, S_g, ds * R, dk, col < dv);
+    const int kvh = MODE == REC_DELTA ? h / (A.nh / A.nkv) : h;
+    float x0[NE], x1[NE], x2[NE], c0[NE], c1[NE];
 #pragma unroll
-        for (int i = 0; i < R; ++i) {
-            const int d = ds * R + i;
-            if (d < dk && col < dv) S_g[d] = S[i];
+    for (int e = 0; e < NE; ++e) {                          // every load first
+        const int d = lane + 64 * e, dd = d < dk ? d : dk - 1;
+        if (MODE == REC_DELTA) {
+            x0[e] = A.q[row * A.ldq + (size_t)kvh * dk + dd];
+            x1[e] = A.k[row * A.ldk + (size_t)kvh * dk + dd];
+            x2[e] = A.dt[row * A.lddt + (size_t)h * dk + dd];
+            c0[e] = A.dt_bias[(size_t)h * dk + dd];
+            c1[e] = 0.f;
+        } else {
+            x0[e] = A.q[row * A.ldq + (size_t)h * dk + dd];
+            x1[e] = A.k[row * A.ldk + (size_t)h * dk + dd];
+            x2[e] = 0.f;
+            c0[e] = A.low[(size_t)h * dk + dd];
+            c1[e] = A.f_bias ? A.f_bias[(size_t)h * dk + dd] : 0.f;
         }
     }
+    float u = A.v[row * A.ldv + (size_t)h * dv + (col < dv ? col : dv - 1)];
+    float beta = 1.f, ea = 0.f;
+    if (MODE == REC_DELTA) {
+        beta = sigmoid_f(A.b[row * A.ldb + h]);
+        ea = expf(A.a_log[h]);
+    }
+    float qi = 1.f, ki = 1.f;
+    if (MODE == REC_DELTA) {
+        float qq = 0.f, kk = 0.f;
+#pragma unroll
+        for (int e = 0; e < NE; ++e)
+            if (lane + 64 * e < dk) { qq = fmaf(x0[e], x0[e], qq); kk = fmaf(x1[e], x1[e], kk); }
+        qq = wave_sum(qq);
+        kk = wave_sum(kk);
+        qi = 1.0f / sqrtf(qq + A.unit_eps) / sqrtf((float)dk);
+        ki = 1.0f / sqrtf(kk + A.unit_eps);
+    }
+    float kq = 0.f;
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        const int d = lane + 64 * e;
+        float a = 0.f, kx = 0.f, qx = 0.f;
+        if (d < dk) {
+            if (MODE == REC_DELTA) {
+                a = expf(-ea * softplus_f(x2[e] + c0[e]));
+                kx = x1[e] * ki;
+                qx = x0[e] * qi;
+            } else {
+                const float f = c0[e] + (1.f - c0[e]) * sigmoid_f(x1[e] + c1[e]);
+                a = f;
+                kx = 1.f - f;
+                qx = silu_f(x0[e]);
+            }
+        }
+        kq = fmaf(kx, qx, kq);
+        if (d < DP) { sa[wv][d] = a; sk[wv][d] = kx; sq[wv][d] = qx; }
+    }
+    kq = wave_sum(kq);
+    __syncthreads();                                        // (a wave reads only what it wrote itself)
+    float dkk = 0.f, dq = 0.f;
+    float kreg[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int d = ds * R + i;
+        kreg[i] = sk[wv][d];
+        S[i] *= sa[wv][d];
+        dq = fmaf(S[i], sq[wv][d], dq);
+        if (MODE == REC_DELTA) dkk = fmaf(S[i], kreg[i], dkk);
+    }
+    dq = lanes_sum<DS>(dq);
+    if (MODE == REC_DELTA) u = beta * (u - lanes_sum<DS>(dkk));
+#pragma unroll
+    for (int i = 0; i < R; ++i) S[i] = fmaf(kreg[i], u, S[i]);
+    state_store<R>(S, S_g, ds * R, dk, col < dv);
+    if (ds == 0 && col < dv) A.o[row * A.ldo + (size_t)h * dv + col] = fmaf(u, kq, dq);
+}
+
+template <int MODE>
+static int launch_recurrence_step(const RecurrenceArgs& A, int n_seqs, hipStream_t stream) {
+    const int cb = A.dk <= 32 ? 64 : 16;
+    const dim3 grid((A.dv + cb - 1) / cb, A.nh, n_seqs);
+    if (A.dk <= 32) gated_recurrence_step_kernel<MODE, 4, 8><<<grid, 256, 0, stream>>>(A);
+    else if (A.dk <= 64) gated_recurrence_step_kernel<MODE, 16, 4><<<grid, 256, 0, stream>>>(A);
+    else if (A.dk <= 128) gated_recurrence_step_kernel<MODE, 16, 8><<<grid, 256, 0, stream>>>(A);
+    else gated_recurrence_step_kernel<MODE, 16, 16><<<grid, 256, 0, stream>>>(A);
+    AGAVE_LAUNCH_CHECK("gated_recurrence_step");
+    return 0;
 }
 
 template <int MODE>
@@ -773,7 +894,7 @@ extern "C" int agave_gated_recurrence(int mode, const float* q, long ldq, const 
                                       const float* dt, long lddt, const float* b, long ldb, const float* a_log,
                                       const float* dt_bias, const float* low, const float* f_bias, float* o, long ldo,
                                       float* state, const int* cu, const int* slots, int n_seqs, int nh, int nkv, int dk,
-                                      int dv, float unit_eps, hipStream_t stream) {
+                                      int dv, float unit_eps, int one_token_each, hipStream_t stream) {
     AGAVE_CHECK(mode == REC_DELTA || mode == REC_FORGET, "gated_recurrence: unknown mode %d", mode);
     AGAVE_CHECK(n_seqs >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "gated_recurrence: bad sizes B=%d nh=%d nkv=%d dk=%d dv=%d", n_seqs, nh, nkv, dk, dv);
     AGAVE_CHECK(dk <= 256, "gated_recurrence: %d key channels a head (up to 256 are supported)", dk);
@@ -790,6 +911,8 @@ extern "C" int agave_gated_recurrence(int mode, const float* q, long ldq, const 
     }
     if (n_seqs == 0) return 0;
     RecurrenceArgs A{q, ldq, k, ldk, v, ldv, dt, lddt, b, ldb, a_log, dt_bias, low, f_bias, o, ldo, state, cu, slots, nh, nkv, dk, dv, unit_eps};
+    if (one_token_each)                                     // the host vouches that every sequence brings one token
+        return mode == REC_DELTA ? launch_recurrence_step<REC_DELTA>(A, n_seqs, stream) : launch_recurrence_step<REC_FORGET>(A, n_seqs, stream);
     return mode == REC_DELTA ? launch_recurrence<REC_DELTA>(A, n_seqs, stream) : launch_recurrence<REC_FORGET>(A, n_seqs, stream);
 }
 

@@ -24,7 +24,7 @@ kernels.register_signatures(LIBRARY, {
     "agave_talk_attention": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I,
                              _F, _I, _F, _P, _I, _P],
     "agave_gated_recurrence": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _P, _L, _P, _P, _P,
-                               _I, _I, _I, _I, _I, _F, _P],
+                               _I, _I, _I, _I, _I, _F, _I, _P],
     "agave_head_norm_gate": [_I, _P, _L, _P, _P, _L, _P, _L, _I, _I, _I, _F, _F, _P],
     "agave_scaled_sum": [_I, _P, _L, _F, _P, _L, _F, _P, _L, _I, _I, _P],
 })
@@ -185,7 +185,7 @@ def gated_recurrence(mode: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     library.call(_lib(), "agave_gated_recurrence", mode, ptr(q), ldq, ptr(k), ldk, ptr(v), ldv, ptr(dt_in), lddt, ptr(beta),
                  ldb, ptr(a_log), ptr(dt_bias), ptr(lower), ptr(f_bias), ptr(out), ldo, ptr(state), ptr(step.cu_dev),
                  ptr(step.slots_dev), step.n_seqs, n_heads, n_kv if mode == DELTA else n_heads, dk, dv, float(unit_eps),
-                 stream())
+                 1 if (step.is_decode and step.n_tokens == step.n_seqs) else 0, stream())
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], out: torch.Tensor,
