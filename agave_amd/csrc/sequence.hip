@@ -251,8 +251,8 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
     }
     __syncthreads();
 
-    // parts: the launch has a workgroup per tile of 64 keys (blockIdx.y), which leaves its sums, maximum and
-    // weight per head for talk_merge_kernel; a tile behind the query's position leaves none (weight 0)
+    // parts: the launch has a workgroup per tile of 64 keys (blockIdx.y) and key head (blockIdx.z), which leaves
+    // its heads' sums, maximum and weight for talk_merge_kernel; a tile behind the query's position leaves none (weight 0)
     const int j_first = parts ? lo + (int)blockIdx.y * 64 : lo;
     const int j_last = parts ? (j_first + 63 < p ? j_first + 63 : p) : p;
     for (int j0 = j_first; j0 <= j_last; j0 += 64) {
@@ -369,7 +369,9 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
         for (int a = 0; a < TALK_ACC; ++a) {
             if (one_h[a] < nh) acc[a] *= alpha[one_h[a]];
         }
-        for (int g = 0; g < nkv; ++g) {
+        // (with parts, a workgroup sums the values of one key head only: blockIdx.z; the scores it needs all)
+        const int g_first = parts ? (int)blockIdx.z : 0, g_end = parts ? g_first + 1 : nkv;
+        for (int g = g_first; g < g_end; ++g) {
             for (int e0 = 0; e0 < dv; e0 += vcols) {
                 const int ec = dv - e0 < vcols ? dv - e0 : vcols;
                 __syncthreads();                                   // the tile before is read
@@ -428,9 +430,10 @@ __global__ __launch_bounds__(256) void talk_attention_kernel(
 #pragma unroll
         for (int a = 0; a < TALK_ACC; ++a) {
             const int h = one_h[a];
-            if (h < nh) mine[(size_t)h * (dv + 2) + (tid + a * 256 - h * dv)] = acc[a];
+            if (h < nh && h / rep == (int)blockIdx.z) mine[(size_t)h * (dv + 2) + (tid + a * 256 - h * dv)] = acc[a];
         }
         for (int h = tid; h < nh; h += 256) {
+            if (h / rep != (int)blockIdx.z) continue;
             mine[(size_t)h * (dv + 2) + dv] = m_run[h];
             mine[(size_t)h * (dv + 2) + dv + 1] = l_run[h];
         }
@@ -494,7 +497,7 @@ extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const f
         vcols, parts, tiles)
     AGAVE_CHECK(!parts || (tiles >= 1 && tiles <= 1024 && chunk > 0 && (long)tiles * 64 >= chunk),
                 "talk_attention: %d tiles of 64 keys do not cover a chunk of %d", tiles, chunk);
-    const dim3 grid(N, parts ? tiles : 1);
+    const dim3 grid(N, parts ? tiles : 1, parts ? nkv : 1);
     const int sums = (nh * dv + 255) / 256;                 // a thread's sums: fewer registers where fewer do
     if (dtype == AGAVE_F32) {
         if (sums <= 4) TALK_LAUNCH(float, 4); else if (sums <= 8) TALK_LAUNCH(float, 8); else TALK_LAUNCH(float, 16);
