@@ -18,9 +18,14 @@
 
 #define CONV_MAX_TAPS 8
 
-__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+// Gates by the hardware's exponential, logarithm and reciprocal (an ulp or two each, absolute errors of
+// about 1e-7 in a gate that lies in (0, 1)): the library's exact versions are 15 to 30 instructions each, and
+// the recurrence's producer waves, which share their SIMDs with the waves that run the chain, spent most of
+// theirs on them.
+__device__ __forceinline__ float sigmoid_f(float x) { return __frcp_rn(1.0f + __expf(-x)); }
 __device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
-__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : __logf(1.0f + __expf(x)); }
+__device__ __forceinline__ float decay_f(float rate, float x) { return __expf(-rate * softplus_f(x)); }
 
 // ------------------------------------------------------------------ short causal convolution
 //   y[t][c] = act(sum_j w[c][j] * u[pos(t) - taps + 1 + j][c]),  zeros before the sequence's start.
@@ -524,7 +529,7 @@ extern "C" int agave_talk_attention(int dtype, const float* q, long ldq, const f
 //     S <- diag(a) S;   u = beta (v - S^T k)  [delta]  or  u = v  [forget gate];   S <- S + k u^T;   o = S^T q
 // so the read-out sees the token's own write.  A column of S (one value element) never meets
 // another: DS lanes share a column's dk rows (R each), a wave owns 64 / DS columns, and the four
-// consumer waves of a workgroup 4 * 64 / DS columns of one head.  Eight producer waves make the gates
+// consumer waves of a workgroup 4 * 64 / DS columns of one head.  Four producer waves make the gates
 // of the next TB tokens into the other half of LDS meanwhile (all their loads asked for before the
 // first is used), so that the chain from token to token never waits for memory:
 //   delta:   q, k: unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times dk^-1/2; key head of h is
@@ -588,12 +593,21 @@ template <int DS> __device__ __forceinline__ float lanes_sum(float v) {
     return v;
 }
 
+// A workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits for every
+// load from memory that is on its way, and the producers' loads for the block after next are meant to stay
+// on their way across it: with the full barrier every block of 16 tokens cost a round trip to memory.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 template <int MODE, int DS, int R, int TB>
-__global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A) {
+__global__ __launch_bounds__(512) void gated_recurrence_kernel(RecurrenceArgs A) {
     constexpr int DP = DS * R;                              // padded rows
     constexpr int CW = 64 / DS, CB = 4 * CW;                // columns a wave, a workgroup
     constexpr int NE = (DP + 63) / 64;                      // elements of a row a producer lane holds
-    constexpr int PW = 8;                                   // producer waves (behind the four consumer waves)
+    constexpr int PW = 4;                                   // producer waves (behind the four consumer waves)
     constexpr int NT = TB / PW;                             // tokens of a block a producer wave makes
     __shared__ __attribute__((aligned(16))) float sa[2][TB][DP];
     __shared__ __attribute__((aligned(16))) float sk[2][TB][DP];
@@ -680,7 +694,7 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
                 float a = real ? 0.f : 1.f, kx = 0.f, qx = 0.f;
                 if (d < dk && real) {
                     if (MODE == REC_DELTA) {
-                        a = expf(-ea * softplus_f(x2[t][e] + c0[e]));
+                        a = decay_f(ea, x2[t][e] + c0[e]);
                         kx = x1[t][e] * ki;
                         qx = x0[t][e] * qi;
                     } else {
@@ -759,7 +773,7 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
         make(0, 0);
         if (n_blocks > 1) ask(1);
     }
-    __syncthreads();
+    lds_barrier();
     for (int blk = 0; blk < n_blocks; ++blk) {
         if (producer) {
             if (blk + 1 < n_blocks) {
@@ -769,14 +783,14 @@ __global__ __launch_bounds__(768) void gated_recurrence_kernel(RecurrenceArgs A)
         } else {
             consume(blk, blk & 1);
         }
-        __syncthreads();                                    // the block just read may be overwritten, the one just made be read
+        lds_barrier();                                      // the block just read may be overwritten, the one just made be read
     }
     if (!producer) state_store<R>(S, S_g, ds * R, dk, col < dv);
 }
 
 // One token per sequence (a decode step): four waves, each with 64 / DS columns, and every wave makes
 // the token's gates for itself, so nothing waits for another wave's work and a compute unit holds eight
-// such workgroups (the kernel above, with its twelve waves, holds one: 1,024 workgroups took four rounds).
+// such workgroups (the kernel above, with its eight waves and two halves of LDS, holds far fewer).
 template <int MODE, int DS, int R>
 __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceArgs A) {
     constexpr int DP = DS * R, CW = 64 / DS, CB = 4 * CW, NE = (DP + 63) / 64;
@@ -834,7 +848,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_step_kernel(RecurrenceAr
         float a = 0.f, kx = 0.f, qx = 0.f;
         if (d < dk) {
             if (MODE == REC_DELTA) {
-                a = expf(-ea * softplus_f(x2[e] + c0[e]));
+                a = decay_f(ea, x2[e] + c0[e]);
                 kx = x1[e] * ki;
                 qx = x0[e] * qi;
             } else {
@@ -885,10 +899,10 @@ static int launch_recurrence(const RecurrenceArgs& A, int n_seqs, hipStream_t st
     // are then made twice instead of eight times, and the step was 6 % slower: the longer chain of a token)
     const int cb = A.dk <= 32 ? 64 : 16;                    // columns a workgroup, as the kernel's CB
     const dim3 grid((A.dv + cb - 1) / cb, A.nh, n_seqs);
-    if (A.dk <= 32) gated_recurrence_kernel<MODE, 4, 8, 16><<<grid, 768, 0, stream>>>(A);
-    else if (A.dk <= 64) gated_recurrence_kernel<MODE, 16, 4, 16><<<grid, 768, 0, stream>>>(A);
-    else if (A.dk <= 128) gated_recurrence_kernel<MODE, 16, 8, 16><<<grid, 768, 0, stream>>>(A);
-    else gated_recurrence_kernel<MODE, 16, 16, 8><<<grid, 768, 0, stream>>>(A);
+    if (A.dk <= 32) gated_recurrence_kernel<MODE, 4, 8, 16><<<grid, 512, 0, stream>>>(A);
+    else if (A.dk <= 64) gated_recurrence_kernel<MODE, 16, 4, 16><<<grid, 512, 0, stream>>>(A);
+    else if (A.dk <= 128) gated_recurrence_kernel<MODE, 16, 8, 16><<<grid, 512, 0, stream>>>(A);
+    else gated_recurrence_kernel<MODE, 16, 16, 8><<<grid, 512, 0, stream>>>(A);
     AGAVE_LAUNCH_CHECK("gated_recurrence");
     return 0;
 }
