@@ -192,7 +192,7 @@ class KVCache:
                     if n > 0:
                         lens[i] += n
                         keep_from = g._first_needed(lens[i])
-                        held[i] = {x for x in held[i] if x >= keep_from}
+                        held[i] = {x for x in held[i] if x >= keep_from or x < g.key.kept_pages}
 
     def commit_step(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
         for s, n in zip(slots, n_new):

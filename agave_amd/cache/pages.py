@@ -107,6 +107,26 @@ class GroupKey:
     # matrix cores' operand order where the sizes allow; "rows": K and V row by row,
     # [page, kv head, 64, head_dim] and [page, kv head, 64, v_head_dim], never reordered
     layout: str = "tiles"
+    # The first positions of a sequence that stay visible whatever the window: the pages that hold them
+    # are never given back, and stand in the first columns of a step's table row (``kept_pages``).
+    keep_first: int = 0
+
+    @property
+    def kept_pages(self) -> int:
+        """Pages at a sequence's start that are held for good (0 without a window: every page is)."""
+        return (self.keep_first + PAGE - 1) // PAGE if (self.keep_first > 0 and self.reach is not None) else 0
+
+    def covering(self, other: "GroupKey") -> Optional["GroupKey"]:
+        """The need that serves this one and ``other`` on the same pages (two mixers that read one memory with
+        different windows): the wider window, the larger count of kept positions.  None if sizes, chunk or
+        layout differ."""
+        same = (self.n_kv_heads, self.head_dim, self.chunk, self.v_head_dim, self.layout) == \
+               (other.n_kv_heads, other.head_dim, other.chunk, other.v_head_dim, other.layout)
+        if not same:
+            return None
+        window = None if (self.window is None or other.window is None) else max(self.window, other.window)
+        return GroupKey(window, self.n_kv_heads, self.head_dim, self.chunk, self.v_head_dim, self.layout,
+                        max(self.keep_first, other.keep_first))
 
     @property
     def reach(self) -> Optional[int]:
@@ -124,23 +144,24 @@ class GroupKey:
         return lo
 
 
-def pages_in_reach(window: Optional[int], max_context: int, max_new: int = 1) -> int:
+def pages_in_reach(window: Optional[int], max_context: int, max_new: int = 1, kept_pages: int = 0) -> int:
     """Most pages one sequence holds in a group while a step brings it up to ``max_new`` tokens,
     for sequences of at most ``max_context`` positions.  A group that needs all keys holds the
     whole context.  A window of W reaches back W - 1 positions from the step's first token, so
-    the step spans W + max_new - 1 positions, which touch at most one page more than they fill."""
+    the step spans W + max_new - 1 positions, which touch at most one page more than they fill.
+    ``kept_pages``: pages at the sequence's start that a windowed group holds besides."""
     full = (max_context + PAGE - 1) // PAGE
     if window is None:
         return full
-    return min(full, (window + max_new - 1 + PAGE - 2) // PAGE + 1)
+    return min(full, (window + max_new - 1 + PAGE - 2) // PAGE + 1 + kept_pages)
 
 
-def pool_pages(window: Optional[int], max_slots: int, max_context: int, piece: int) -> int:
+def pool_pages(window: Optional[int], max_slots: int, max_context: int, piece: int, kept_pages: int = 0) -> int:
     """Pages a group's pool needs so that ``max_slots`` sequences of up to ``max_context``
     positions always fit when no step brings a sequence more than ``piece`` tokens: all keys of
     every sequence for a group without a window, only the window's reach plus the step's own
     tokens for a windowed one (what the reference's ring of W rows per sliding layer bounds)."""
-    return max_slots * pages_in_reach(window, max_context, max(1, min(piece, max_context)))
+    return max_slots * pages_in_reach(window, max_context, max(1, min(piece, max_context)), kept_pages)
 
 
 class GroupPages:
@@ -159,12 +180,14 @@ class GroupPages:
     def table_width(self, max_context: int, max_new: int = 1) -> int:
         """Columns that a step's table needs at most for sequences up to ``max_context``
         positions when a step brings up to ``max_new`` tokens per sequence."""
-        return pages_in_reach(self.key.reach, max_context, max_new)
+        return pages_in_reach(self.key.reach, max_context, max_new, self.key.kept_pages)
 
     def plan(self, slot: int, pos0: int, n_new: int) -> Tuple[int, List[int]]:
         """Make sure pages exist for positions ``pos0 .. pos0+n_new-1`` and return
         ``(base, pages)``: ``pages[i]`` is the page id of page index ``base + i``, from the
-        oldest page a query of this step can reach to the newest page it writes."""
+        oldest page a query of this step can reach to the newest page it writes.  In a group that
+        keeps a sequence's first pages (``key.kept_pages`` = k > 0) those come first: ``pages[i]`` is
+        page index i for i < k, and page index ``base + i - k`` from there on, with ``base >= k``."""
         if n_new < 1:
             raise CacheError("a step brings at least one token per sequence")
         held = self._pages[slot]
@@ -175,17 +198,20 @@ class GroupPages:
                              f"of {self.pool.n_pages}")
         for i in fresh:
             held[i] = self.pool.alloc()
-        base = self._first_needed(pos0)
-        missing = [i for i in range(base, last_new + 1) if i not in held]
+        kept = self.key.kept_pages
+        base = max(self._first_needed(pos0), kept)
+        wanted = list(range(0, min(kept, last_new + 1))) + list(range(base, last_new + 1))
+        missing = [i for i in wanted if i not in held]
         if missing:
             raise CacheError(f"slot {slot}: pages {missing} within reach are not held")
-        return base, [held[i] for i in range(base, last_new + 1)]
+        return base, [held[i] for i in wanted]
 
     def commit(self, slot: int, new_length: int) -> None:
         """After a step: give back the pages that no later query reaches."""
         held = self._pages[slot]
         keep_from = self._first_needed(new_length)
-        for i in [i for i in held if i < keep_from]:
+        kept = self.key.kept_pages
+        for i in [i for i in held if kept <= i < keep_from]:
             self.pool.free(held.pop(i))
 
     def release(self, slot: int) -> None:

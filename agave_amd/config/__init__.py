@@ -1,10 +1,11 @@
 """Typed configurations and the architecture registry."""
 from .errors import ConfigError, UnsupportedArchitecture
 from .gemma3 import Gemma3Config
+from .gusedra import GusedraConfig
 from .registry import (Architecture, architectures, find_architecture, load_config,
                        read_config_json, register_architecture)
 from .rilenex import RilenexConfig
-from .spec import (AttentionSpec, DenseFfnSpec, FeedForwardSpec, GatedDeltaSpec, GatedFfnSpec, Hgrn2Spec, LayerSpec,
+from .spec import (AttentionSpec, BiasedAttentionSpec, RoutedFfnSpec, ScoreBiasSpec, DenseFfnSpec, FeedForwardSpec, GatedDeltaSpec, GatedFfnSpec, Hgrn2Spec, LayerSpec,
                    MixerSpec, ModelSpec, NormSpec, ParallelMixerSpec, PositionSpec, RunEntry, TalkingAttentionSpec)
 
 register_architecture(Architecture(
@@ -19,8 +20,14 @@ register_architecture(Architecture(
     parse=RilenexConfig.from_dict,
     spec=lambda cfg, names=None: cfg.model_spec(names)))
 
+register_architecture(Architecture(
+    name=GusedraConfig.architecture,
+    model_types=("gusedra",),
+    parse=GusedraConfig.from_dict,
+    spec=lambda cfg, names=None: cfg.model_spec(names)))
+
 __all__ = [
-    "ConfigError", "UnsupportedArchitecture", "Gemma3Config", "RilenexConfig", "Architecture", "architectures",
+    "ConfigError", "UnsupportedArchitecture", "Gemma3Config", "RilenexConfig", "GusedraConfig", "BiasedAttentionSpec", "RoutedFfnSpec", "ScoreBiasSpec", "Architecture", "architectures",
     "find_architecture", "load_config", "read_config_json", "register_architecture",
     "AttentionSpec", "FeedForwardSpec", "GatedFfnSpec", "LayerSpec", "MixerSpec", "ModelSpec",
     "NormSpec", "PositionSpec", "RunEntry", "TalkingAttentionSpec", "GatedDeltaSpec", "Hgrn2Spec",

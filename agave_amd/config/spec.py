@@ -16,11 +16,14 @@ from typing import Dict, List, Optional, Tuple
 @dataclass(frozen=True)
 class NormSpec:
     """A normalisation over the last axis.  ``weight`` is the tensor's full name."""
-    kind: str                      # "rmsnorm"
+    kind: str                      # "rmsnorm" | "layernorm"
     size: int
     eps: float
     weight: str
     add_one: bool = False          # gain = 1 + w instead of w
+    bias: str = ""                 # layernorm: the tensor added after the weight; "": none
+    scale_by: str = ""             # a vector that multiplies the norm's result element by element (a layer scale); "": none
+    mult: float = 1.0              # a number that multiplies the norm's result (a multiplier on a residual branch)
 
 
 @dataclass(frozen=True)
@@ -85,6 +88,43 @@ class TalkingAttentionSpec(MixerSpec):
     v_conv: str = ""
     talk: str = ""                 # [heads, heads]: score_h <- sum_g talk[h, g] score_g; "": none
     gate_proj: str = ""            # [heads, hidden]: head h's output times sigmoid(gate_proj x)_h; "": none
+
+
+@dataclass(frozen=True)
+class ScoreBiasSpec:
+    """What is added to an attention score as a function of the distance n = i - j between query and key.
+
+    ``"none"``;  ``"slopes"``: -slope_h n with slope_h = 2^(-slope_log2 (h + 1) / heads);
+    ``"buckets"``: table[bucket(n), h] for a learned table of B rows, with
+    bucket(n) = n for n < B // 2, else min(B - 1, B // 2 + floor(ln(n / (B // 2)) / ln(max_distance / (B // 2)) (B - B // 2)))."""
+    kind: str = "none"
+    slope_log2: float = 8.0
+    table: str = ""                # [buckets, heads]
+    buckets: int = 0
+    max_distance: int = 0
+
+
+@dataclass(frozen=True)
+class BiasedAttentionSpec(MixerSpec):
+    """Softmax attention without a rotation whose scores get a bias by distance, with keys and values of
+    different sizes, a window, first positions that stay visible, an optional sink in the softmax's
+    denominator and an optional sigmoid gate on the concatenated heads.  Without ``k_proj`` and ``v_proj``
+    the mixer has no keys and values of its own and reads the memory its run-order entry names."""
+    hidden: int = 0
+    n_heads: int = 0
+    n_kv_heads: int = 0
+    head_dim: int = 0              # queries and keys
+    v_head_dim: int = 0            # values
+    scale: float = 1.0             # multiplies q.k (not the bias)
+    window: Optional[int] = None   # None: all earlier keys; W: keys i-W+1 .. i
+    keep_first: int = 0            # keys j < keep_first stay visible whatever the window
+    bias: ScoreBiasSpec = ScoreBiasSpec()
+    sink: str = ""                 # [heads]: exp(sink_h) joins the denominator; "": none
+    gate_proj: str = ""            # [heads * v_head_dim, hidden]: heads times sigmoid(gate_proj x); "": none
+    q_proj: str = ""
+    k_proj: str = ""
+    v_proj: str = ""
+    o_proj: str = ""
 
 
 @dataclass(frozen=True)
@@ -169,6 +209,32 @@ class GatedFfnSpec(FeedForwardSpec):
     gate_bias: str = ""            # names of the products' bias vectors; "": none
     up_bias: str = ""
     down_bias: str = ""
+
+
+@dataclass(frozen=True)
+class RoutedFfnSpec(FeedForwardSpec):
+    """A mixture of gated experts ``W_down (act(W_gate x) * (W_up x))``.  The router has ``n_experts +
+    n_identity`` outputs; the last ``n_identity`` stand for experts whose result is their input.  Scores are
+    the softmax over all outputs; the ``top`` outputs with the largest score + correction are chosen, among
+    the ``keep_groups`` best of ``groups`` equal groups of neighbouring outputs (a group counts by its largest
+    score + correction); a chosen expert's weight is its score times ``route_scale``.  ``shared``: an expert
+    that every token runs through, added."""
+    hidden: int = 0
+    intermediate: int = 0          # of every expert
+    n_experts: int = 0
+    n_identity: int = 0
+    top: int = 1
+    groups: int = 1
+    keep_groups: int = 1
+    route_scale: float = 1.0
+    activation: str = "silu"
+    router: str = ""               # [n_experts + n_identity, hidden]
+    correction: str = ""           # [n_experts + n_identity]; "": none
+    expert_prefix: str = ""        # expert i's matrices are expert_prefix + f"{i}." + gate | up | down
+    gate_name: str = "gate"
+    up_name: str = "up"
+    down_name: str = "down"
+    shared: Optional[GatedFfnSpec] = None
 
 
 @dataclass(frozen=True)

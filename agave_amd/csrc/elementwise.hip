@@ -298,6 +298,107 @@ extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long
     return 0;
 }
 
+// ------------------------------------------------------------------ residual + layer norms
+// The same two steps with norms that subtract the mean and have a weight and a bias:
+//   ln(v) = (v - mean(v)) / sqrt(mean((v - mean(v))^2) + eps) * w + b
+//   if branch: h[r] += post_w ? ln_post(branch[r]) : branch[r]
+//   if out:    out[i] = ln_pre(h[r])
+// Mean and variance are taken in two passes over the row, which waits in LDS (e floats).
+template <typename T>
+__global__ void residual_layernorm_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
+                                          long part_stride, const float* __restrict__ post_w, const float* __restrict__ post_b,
+                                          float post_eps, T* __restrict__ out, long ldo, const float* __restrict__ pre_w,
+                                          const float* __restrict__ pre_b, float pre_eps, const int* __restrict__ rows, int e,
+                                          const float* __restrict__ h_src) {
+    extern __shared__ float row[];
+    __shared__ float red[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    float* hr = h + (size_t)r * e;
+    const float* hs = h_src ? h_src + (size_t)r * e : hr;
+    if (branch) {
+        const T* br = branch + (size_t)r * ldb;
+        const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb;
+        float sum = 0.f;
+        for (int c = threadIdx.x; c < e; c += blockDim.x) {
+            float v;
+            if (n_parts == 0) {
+                v = ld(br + c);
+            } else {
+                v = 0.f;
+                for (int p = 0; p < n_parts; ++p) v += parts[(size_t)p * part_stride + c];
+            }
+            row[c] = v;
+            sum += v;
+        }
+        float mean = 0.f, inv = 1.f;
+        if (post_w) {
+            mean = block_sum(sum, red) / (float)e;
+            float sq = 0.f;
+            for (int c = threadIdx.x; c < e; c += blockDim.x) {
+                const float d = row[c] - mean;
+                sq += d * d;
+            }
+            inv = 1.0f / sqrtf(block_sum(sq, red) / (float)e + post_eps);
+        }
+        for (int c = threadIdx.x; c < e; c += blockDim.x) {
+            const float y = post_w ? (row[c] - mean) * inv * post_w[c] + (post_b ? post_b[c] : 0.f) : row[c];
+            const float hv = hs[c] + y;
+            hr[c] = hv;
+            row[c] = hv;
+        }
+    } else {
+        for (int c = threadIdx.x; c < e; c += blockDim.x) {
+            const float hv = hs[c];
+            if (h_src) hr[c] = hv;
+            row[c] = hv;
+        }
+    }
+    if (out) {
+        float sum = 0.f;
+        for (int c = threadIdx.x; c < e; c += blockDim.x) sum += row[c];
+        const float mean = block_sum(sum, red) / (float)e;
+        float sq = 0.f;
+        for (int c = threadIdx.x; c < e; c += blockDim.x) {
+            const float d = row[c] - mean;
+            sq += d * d;
+        }
+        const float inv = 1.0f / sqrtf(block_sum(sq, red) / (float)e + pre_eps);
+        T* o = out + (size_t)i * ldo;
+        for (int c = threadIdx.x; c < e; c += blockDim.x) st(o + c, (row[c] - mean) * inv * pre_w[c] + (pre_b ? pre_b[c] : 0.f));
+    }
+}
+
+// The arguments are residual_norm's, with a bias beside each weight (null: none).
+extern "C" int agave_residual_layernorm(int dtype, float* h, const void* branch, long ldb, int n_parts, long part_stride,
+                                        const float* post_w, const float* post_b, float post_eps, void* out, long ldo,
+                                        const float* pre_w, const float* pre_b, float pre_eps, const int* rows, int n_rows,
+                                        int e, const float* h_src, hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && e > 0 && e <= 15360, "residual_layernorm: bad sizes rows=%d e=%d (rows of up to 15360)", n_rows, e);
+    AGAVE_CHECK(h != nullptr, "residual_layernorm: residual stream is null");
+    AGAVE_CHECK(!(h_src && rows), "residual_layernorm: rows are gathered from the residual stream itself");
+    AGAVE_CHECK(!out || pre_w, "residual_layernorm: output without its weight");
+    AGAVE_CHECK(!branch || ldb >= e, "residual_layernorm: branch row stride %ld < %d", ldb, e);
+    AGAVE_CHECK(!out || ldo >= e, "residual_layernorm: output row stride %ld < %d", ldo, e);
+    AGAVE_CHECK(!(rows && branch), "residual_layernorm: row gather with a branch is not supported");
+    AGAVE_CHECK(n_parts >= 0 && n_parts <= 64 && (n_parts == 0 || branch), "residual_layernorm: %d slices", n_parts);
+    if (n_rows == 0 || (!branch && !out && !h_src)) return 0;
+    const int threads = e >= 2048 ? 512 : (e >= 512 ? 256 : 64);
+    const size_t lds = (size_t)e * sizeof(float);
+    if (dtype == AGAVE_F32)
+        residual_layernorm_kernel<float><<<n_rows, threads, lds, stream>>>(h, (const float*)branch, ldb, n_parts, part_stride, post_w,
+                                                                           post_b, post_eps, (float*)out, ldo, pre_w, pre_b,
+                                                                           pre_eps, rows, e, h_src);
+    else if (dtype == AGAVE_BF16)
+        residual_layernorm_kernel<bf16><<<n_rows, threads, lds, stream>>>(h, (const bf16*)branch, ldb, n_parts, part_stride, post_w,
+                                                                          post_b, post_eps, (bf16*)out, ldo, pre_w, pre_b,
+                                                                          pre_eps, rows, e, h_src);
+    else
+        AGAVE_CHECK(false, "residual_layernorm: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("residual_layernorm");
+    return 0;
+}
+
 // ------------------------------------------------------------------ q/k head norm + rotation + cache write
 // One wave per (token, head); q heads first, then k heads.  A k-head wave also stores the
 // matching v head.  Cache pages: K [page][kv head][64 rows][hd], V transposed
@@ -489,10 +590,12 @@ extern "C" int agave_gated_act(int dtype, int act, const void* gate, long ldg, c
 // (the tanh form of gelu under its older name)
 // ------------------------------------------------------------------ an activation on its own
 // out = act(x) for a feed-forward without a gate.  Activations 0 to 3 are the gate's; 4 is xIELU with
-// its two factors made by the host:  x > 0: ap x^2 + x/2;  x <= 0: an (exp(x) - 1 - x) + x/2.
-#define AGAVE_UNARY_ACTS 5
+// its two factors made by the host:  x > 0: ap x^2 + x/2;  x <= 0: an (exp(x) - 1 - x) + x/2;
+// 5 is the square of relu.
+#define AGAVE_UNARY_ACTS 6
 __device__ __forceinline__ float unary_act_value(float z, int act, float p0, float p1) {
     if (act == 4) return z > 0.f ? fmaf(p0 * z, z, 0.5f * z) : fmaf(p1, expm1f(z) - z, 0.5f * z);
+    if (act == 5) return z > 0.f ? z * z : 0.f;
     return gate_act(z, act);
 }
 

@@ -112,7 +112,7 @@ class Engine:
         pages: Dict[GroupKey, int] = {}
         for key in set(kv_needs.values()):
             # what max_slots sequences can hold at most; fewer if the caller bounds the live positions
-            pages[key] = pool_pages(key.reach, max_slots, self.max_context, self.max_piece)
+            pages[key] = pool_pages(key.reach, max_slots, self.max_context, self.max_piece, key.kept_pages)
             if cache_tokens is not None:
                 pages[key] = min(pages[key], max(1, (int(cache_tokens) + PAGE - 1) // PAGE))
         self.cache = KVCache(kv_needs, self.model.state_needs(), max_slots, pages, self.dtype, self.device,

@@ -65,8 +65,12 @@ class Model:
             if need is None:
                 continue
             if e.memory in needs and needs[e.memory] != need:
-                raise ValueError(f"memory {e.memory} is shared by mixers with different needs: "
-                                 f"{needs[e.memory]} and {need}")
+                # two mixers that read one memory through different windows: the pages serve the wider one
+                both = needs[e.memory].covering(need)
+                if both is None:
+                    raise ValueError(f"memory {e.memory} is shared by mixers with different needs: "
+                                     f"{needs[e.memory]} and {need}")
+                need = both
             needs[e.memory] = need
         return needs
 

@@ -1,0 +1,97 @@
+"""Python faces of ``csrc/attention_biased.hip``: attention over cache pages stored row by row with a
+bias on the scores that depends on the distance between query and key, a window with first
+positions that stay visible, a sink in the softmax's denominator, and a gate on the output rows.
+
+Every function checks on the host what its kernel and grid assume and launches on the current stream.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import kernels, library
+from .kernels import _P, _I, _L, _F, _dev, _f32vec, _i32, _rows, dt, ptr, stream
+
+LIBRARY = "attention_biased"
+
+BIAS_NONE, BIAS_SLOPES, BIAS_TABLE = 0, 1, 2
+
+kernels.register_signatures(LIBRARY, {
+    "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P],
+    "agave_attn_biased_plain": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F,
+                                _I, _I, _I, _P, _I, _P, _P],
+})
+
+
+def _lib():
+    return kernels.lib(LIBRARY)
+
+
+def _check_row_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, vd: int, dtype: torch.dtype) -> int:
+    if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd) or not k_pages.is_contiguous():
+        raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd}], got {tuple(k_pages.shape)}")
+    if v_pages.dim() != 4 or tuple(v_pages.shape[1:]) != (nkv, 64, vd) or not v_pages.is_contiguous():
+        raise ValueError(f"V pages must be contiguous [pages, {nkv}, 64, {vd}], got {tuple(v_pages.shape)}")
+    if k_pages.shape[0] != v_pages.shape[0] or k_pages.dtype != dtype or v_pages.dtype != dtype:
+        raise ValueError("K and V pages must agree in page count and dtype with the activations")
+    return k_pages.shape[0]
+
+
+def _check_table(table: torch.Tensor, base: torch.Tensor, head: int, keep_first: int) -> int:
+    width = kernels._check_table(table, base, None)
+    if head < 0 or keep_first < 0 or keep_first > head * 64:
+        raise ValueError(f"{keep_first} kept first positions need {-(-keep_first // 64)} kept pages, the table has {head}")
+    return width
+
+
+def kv_append_rows(k: torch.Tensor, v: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, table: torch.Tensor,
+                   base: torch.Tensor, head: int, step, n_kv: int, head_dim: int, v_head_dim: int) -> None:
+    """The step's key and value rows into their places in the cache pages (row by row, as they are)."""
+    _dev(k, v, k_pages, v_pages, table, base)
+    n = step.n_tokens
+    ldk, ldv = _rows(k, "k"), _rows(v, "v")
+    if k.shape != (n, n_kv * head_dim) or v.shape != (n, n_kv * v_head_dim) or k.dtype != v.dtype:
+        raise ValueError(f"k and v must be [{n}, {n_kv * head_dim}] and [{n}, {n_kv * v_head_dim}] of one dtype")
+    n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, k.dtype)
+    width = _check_table(table, base, head, 0)
+    library.call(_lib(), "agave_kv_append_rows", dt(k), ptr(k), ldk, ptr(v), ldv, ptr(k_pages), ptr(v_pages), ptr(table),
+                 width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n, n_kv, head_dim, v_head_dim,
+                 stream())
+
+
+def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torch.Tensor,
+              v_pages: torch.Tensor, table: torch.Tensor, base: torch.Tensor, head: int, step, n_heads: int, n_kv: int,
+              head_dim: int, v_head_dim: int, scale: float, window: Optional[int], keep_first: int, bias_mode: int,
+              bias: Optional[torch.Tensor], sink: Optional[torch.Tensor]) -> None:
+    """out[t, h] = sum_j w_j v_j with w = softmax_j(scale q.k_j + bias(h, p - j)) over the keys that token t at
+    position p sees (j <= p and (p - j < window or j < keep_first)), the sink's exp(sink_h) added to the
+    denominator, times sigmoid(gate[t, h]) element by element.  ``bias``: slopes [heads] (``BIAS_SLOPES``:
+    the bias is -slope_h (p - j)) or a table [heads, distances] (``BIAS_TABLE``: distances beyond the table take
+    its last column)."""
+    _dev(q, out, gate, k_pages, v_pages, table, base, bias, sink)
+    n = step.n_tokens
+    ldq, ldo = _rows(q, "q"), _rows(out, "out")
+    if q.shape != (n, n_heads * head_dim) or out.shape != (n, n_heads * v_head_dim) or out.dtype != q.dtype:
+        raise ValueError(f"attention: q must be [{n}, {n_heads * head_dim}] and out [{n}, {n_heads * v_head_dim}] of one dtype")
+    ldg = 0
+    if gate is not None:
+        ldg = _rows(gate, "gate")
+        if gate.shape != out.shape or gate.dtype != q.dtype:
+            raise ValueError("attention: the gate must have the output's shape and dtype")
+    n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, q.dtype)
+    width = _check_table(table, base, head, keep_first)
+    bias_len = 0
+    if bias_mode == BIAS_SLOPES:
+        _f32vec(bias, "slopes", n_heads)
+    elif bias_mode == BIAS_TABLE:
+        if bias is None or bias.dtype != torch.float32 or bias.dim() != 2 or bias.shape[0] != n_heads or not bias.is_contiguous():
+            raise ValueError(f"attention: the bias table must be contiguous float32 [{n_heads}, distances]")
+        bias_len = bias.shape[1]
+    elif bias_mode != BIAS_NONE:
+        raise ValueError(f"attention: unknown bias mode {bias_mode}")
+    _f32vec(sink, "sink", n_heads)
+    library.call(_lib(), "agave_attn_biased_plain", dt(q), ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages),
+                 ptr(v_pages), ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n,
+                 n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0), int(keep_first), bias_mode,
+                 ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), stream())

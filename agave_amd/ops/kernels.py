@@ -22,6 +22,7 @@ _SIGNATURES = {
     "elementwise": {
         "agave_embed_scale": [_I, _P, _P, _F, _P, _I, _I, _I, _P],
         "agave_residual_norm": [_I, _P, _P, _L, _I, _L, _P, _F, _P, _L, _P, _F, _P, _I, _I, _P, _P],
+        "agave_residual_layernorm": [_I, _P, _P, _L, _I, _L, _P, _P, _F, _P, _L, _P, _P, _F, _P, _I, _I, _P, _P],
         "agave_qk_norm_rope_kv": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F,
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
@@ -177,6 +178,57 @@ def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Op
                  ptr(post_gain), post_eps, ptr(out), ldo, ptr(pre_gain), pre_eps, ptr(rows), n, e, ptr(src), stream())
 
 
+def residual_layernorm(h: torch.Tensor, branch: Optional[torch.Tensor], post_w: Optional[torch.Tensor],
+                       post_b: Optional[torch.Tensor], post_eps: float, out: Optional[torch.Tensor],
+                       pre_w: Optional[torch.Tensor], pre_b: Optional[torch.Tensor], pre_eps: float,
+                       rows: Optional[torch.Tensor] = None, src: Optional[torch.Tensor] = None) -> None:
+    """:func:`residual_norm` with layer norms, ``ln(v) = (v - mean) / sqrt(var + eps) * w + b`` (the variance
+    is the mean of the squared deviations; a bias may be None).  If ``branch``: h += ln_post(branch) (h += branch
+    without ``post_w``).  If ``out``: out = ln_pre(h).  ``rows``, ``src`` and a branch of 32-bit slices as there."""
+    _dev(h, branch, post_w, post_b, out, pre_w, pre_b, rows, src)
+    if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+        raise ValueError("residual stream must be a contiguous float32 [rows, hidden] tensor")
+    n_h, e = h.shape
+    n = n_h if rows is None else rows.numel()
+    _i32(rows, "rows")
+    if src is not None:
+        if src.dtype != torch.float32 or src.shape != h.shape or not src.is_contiguous() or src.data_ptr() == h.data_ptr():
+            raise ValueError("the source of the residual rows must be another contiguous float32 tensor of h's shape")
+        if rows is not None:
+            raise ValueError("rows are gathered from the residual stream itself, not from another source")
+    if rows is not None and branch is not None:
+        raise ValueError("residual_layernorm: rows are gathered only without a branch")
+    act = branch if branch is not None else out
+    if act is None:
+        if src is not None:
+            h.copy_(src)
+        return
+    ldb = ldo = n_parts = part_stride = 0
+    if branch is not None and branch.dim() == 3:
+        if branch.dtype != torch.float32 or branch.shape[1:] != (n_h, e) or not branch.is_contiguous():
+            raise ValueError(f"partial sums must be a contiguous float32 [slices, {n_h}, {e}] tensor")
+        n_parts, part_stride, ldb = branch.shape[0], n_h * e, e
+        if out is not None:
+            act = out
+    elif branch is not None:
+        ldb = _rows(branch, "branch")
+        if branch.shape != (n_h, e):
+            raise ValueError(f"branch must be [{n_h}, {e}], got {tuple(branch.shape)}")
+    for name, v in (("post_w", post_w), ("post_b", post_b), ("pre_w", pre_w), ("pre_b", pre_b)):
+        _f32vec(v, name, e)
+    if out is not None:
+        ldo = _rows(out, "out")
+        if out.shape != (n, e):
+            raise ValueError(f"out must be [{n}, {e}], got {tuple(out.shape)}")
+        if pre_w is None:
+            raise ValueError("residual_layernorm: an output needs its norm's weight")
+        if branch is not None and n_parts == 0 and branch.dtype != out.dtype:
+            raise TypeError("branch and out must have the same dtype")
+    library.call(lib("elementwise"), "agave_residual_layernorm", dt(act), ptr(h), ptr(branch), ldb, n_parts, part_stride,
+                 ptr(post_w), ptr(post_b), post_eps, ptr(out), ldo, ptr(pre_w), ptr(pre_b), pre_eps, ptr(rows), n, e,
+                 ptr(src), stream())
+
+
 def qk_norm_rope_kv(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Optional[torch.Tensor],
                     q_out: Optional[torch.Tensor], q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor],
                     eps_q: float, eps_k: float, inv_freq: Optional[torch.Tensor], pos_scale: float,
@@ -259,8 +311,8 @@ def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activatio
                  stream())
 
 
-# The activations of a feed-forward without a gate: the gate's, and xIELU with two learned numbers.
-UNARY_ACTIVATIONS = dict(GATE_ACTIVATIONS, xielu=4)
+# The activations of a feed-forward without a gate: the gate's, xIELU with two learned numbers, and the square of ReLU.
+UNARY_ACTIVATIONS = dict(GATE_ACTIVATIONS, xielu=4, relu2=5)
 
 
 def unary_act(x: torch.Tensor, out: torch.Tensor, activation: str, p0: float = 0.0, p1: float = 0.0) -> None:

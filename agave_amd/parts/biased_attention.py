@@ -1,0 +1,150 @@
+"""Softmax attention with a bias on the scores by distance, as a mixer.
+
+In the order of its steps: q, k, v (and the gate's logits) in one product; k and v rows appended to
+the cache as they are (there is no rotation and no norm: positions enter through the bias and the
+mask alone); scores ``scale * q.k`` plus the bias of the distance ``i - j``; the keys ``j <= i`` with
+``i - j < window`` or ``j < keep_first``; softmax, with ``exp(sink_h)`` added to the denominator where the
+mixer has sinks; the heads' outputs times ``sigmoid(gate)`` element by element where it has a gate; the
+output product.
+
+The bias is either a slope per head (``-slope_h (i - j)``) or a learned table over buckets of distances;
+the buckets are folded into a table over distances once at load (one column per distance up to the one
+from which the last bucket holds), so the kernels know a slope or a table and nothing of buckets.
+
+A mixer without key and value projections appends nothing and reads the memory that its run-order
+entry names (another layer's keys and values as the cache holds them), through its own mask.
+
+Scores, bias, softmax and the sums over the values are 32-bit in both engines.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional
+
+import torch
+
+from ..cache import GroupKey, StateNeed
+from ..config.spec import BiasedAttentionSpec, ScoreBiasSpec
+from ..ops import attention_biased as ops
+from ..weights.loader import TensorNeed
+from .base import BuildEnv, register
+from .linear import Linear
+
+
+def bucket_of_distance(n: int, buckets: int, max_distance: int) -> int:
+    """Distances below half the buckets have a bucket each; beyond, buckets grow evenly in the logarithm of
+    the distance up to ``max_distance``, and the last bucket takes everything farther.  The logarithms are
+    taken in double precision; a quotient within 1e-9 of a whole number counts as that number."""
+    half = buckets // 2
+    if n < half:
+        return n
+    x = math.log(n / half) / math.log(max_distance / half) * (buckets - half)
+    near = round(x)
+    steps = near if abs(x - near) < 1e-9 else math.floor(x)
+    return min(buckets - 1, half + int(steps))
+
+
+def distance_table(table: torch.Tensor, buckets: int, max_distance: int) -> torch.Tensor:
+    """[heads, distances] float32 from a learned [buckets, heads]: column n holds the bias of distance n, the
+    last column that of every distance from there on."""
+    half = buckets // 2
+    if half < 1 or max_distance <= half:
+        raise ValueError(f"a bias over {buckets} buckets needs a largest distance above {half}, got {max_distance}")
+    last = 0
+    while bucket_of_distance(last, buckets, max_distance) < buckets - 1:
+        last += 1
+        if last > max(max_distance, buckets) + 1:
+            raise ValueError("the buckets of distances never reach the last one")
+    idx = torch.tensor([bucket_of_distance(n, buckets, max_distance) for n in range(last + 1)], dtype=torch.long)
+    return table.to(torch.float32)[idx].t().contiguous()
+
+
+class BiasedAttention:
+    @staticmethod
+    def kernel_libraries(spec, dtype):
+        return ("attention_biased",)
+
+    def __init__(self, spec: BiasedAttentionSpec, weights, env: BuildEnv):
+        s = spec
+        if s.n_heads % s.n_kv_heads:
+            raise ValueError("query heads must be a multiple of kv heads")
+        if bool(s.k_proj) != bool(s.v_proj):
+            raise ValueError("biased attention: key and value projections come together or not at all")
+        self.spec, self.env = spec, env
+        self.qd, self.kd, self.vd = s.n_heads * s.head_dim, s.n_kv_heads * s.head_dim, s.n_kv_heads * s.v_head_dim
+        self.ctx = s.n_heads * s.v_head_dim
+        self.own_kv = bool(s.k_proj)
+        mats = [weights.get(s.q_proj)]
+        bounds = [0, self.qd]
+        if self.own_kv:
+            mats += [weights.get(s.k_proj), weights.get(s.v_proj)]
+            bounds += [bounds[-1] + self.kd, bounds[-1] + self.kd + self.vd]
+        if s.gate_proj:
+            mats.append(weights.get(s.gate_proj))
+            bounds.append(bounds[-1] + self.ctx)
+        self._bounds = tuple(bounds)
+        self.proj = Linear(mats, env, "qkvg")          # one product for everything that reads the mixer's input
+        self.o = Linear([weights.get(s.o_proj)], env, "attn_o")
+        self.sink = weights.get(s.sink).to(torch.float32).contiguous().to(env.device) if s.sink else None
+        b = s.bias
+        if b.kind == "none":
+            self.bias_mode, self.bias = ops.BIAS_NONE, None
+        elif b.kind == "slopes":
+            slopes = [2.0 ** (-b.slope_log2 * (h + 1) / s.n_heads) for h in range(s.n_heads)]
+            self.bias_mode, self.bias = ops.BIAS_SLOPES, torch.tensor(slopes, dtype=torch.float32, device=env.device)
+        elif b.kind == "buckets":
+            self.bias_mode = ops.BIAS_TABLE
+            self.bias = distance_table(weights.get(b.table), b.buckets, b.max_distance).to(env.device)
+        else:
+            raise ValueError(f"biased attention: unknown kind of bias {b.kind!r} (none, slopes, buckets)")
+
+    @staticmethod
+    def tensor_needs(spec: BiasedAttentionSpec) -> List[TensorNeed]:
+        s = spec
+        qd, kd, vd, ctx = s.n_heads * s.head_dim, s.n_kv_heads * s.head_dim, s.n_kv_heads * s.v_head_dim, s.n_heads * s.v_head_dim
+        needs = [TensorNeed(s.q_proj, (qd, s.hidden))]
+        if s.k_proj:
+            needs += [TensorNeed(s.k_proj, (kd, s.hidden)), TensorNeed(s.v_proj, (vd, s.hidden))]
+        if s.bias.kind == "buckets":
+            needs.append(TensorNeed(s.bias.table, (s.bias.buckets, s.n_heads)))
+        if s.sink:
+            needs.append(TensorNeed(s.sink, (s.n_heads,)))
+        if s.gate_proj:
+            needs.append(TensorNeed(s.gate_proj, (ctx, s.hidden)))
+        needs.append(TensorNeed(s.o_proj, (s.hidden, ctx)))
+        return needs
+
+    def kv_need(self) -> Optional[GroupKey]:
+        s = self.spec
+        return GroupKey(s.window, s.n_kv_heads, s.head_dim, v_head_dim=s.v_head_dim, layout="rows",
+                        keep_first=s.keep_first if s.window is not None else 0)
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, x: torch.Tensor, step, memory: int, writes: bool = True) -> torch.Tensor:
+        s, ws = self.spec, self.env.workspace
+        n = x.shape[0]
+        if writes != self.own_kv:
+            raise ValueError("biased attention: a mixer with key and value projections appends to its memory, one "
+                             "without reads another's; the run order says otherwise")
+        group = step.cache.group_of_memory[memory]
+        k_pages, v_pages, _ = step.cache.pages_of(memory)
+        table, base = step.tables[group]
+        head = step.cache.group_keys[group].kept_pages
+        proj = self.proj.forward(x, tag="qkvg")
+        cols = ws.columns(proj, self._bounds)
+        q = cols[0]
+        at = 1
+        if self.own_kv:
+            ops.kv_append_rows(cols[1], cols[2], k_pages, v_pages, table, base, head, step, s.n_kv_heads, s.head_dim,
+                               s.v_head_dim)
+            at = 3
+        gate = cols[at] if s.gate_proj else None
+        ctx = ws.get("attn_ctx", n, self.ctx, x.dtype)
+        ops.attention(q, ctx, gate, k_pages, v_pages, table, base, head, step, s.n_heads, s.n_kv_heads, s.head_dim,
+                      s.v_head_dim, s.scale, s.window, s.keep_first, self.bias_mode, self.bias, self.sink)
+        return self.o.forward(ctx, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream
+
+
+register("mixer", "biased_attention", BiasedAttention)

@@ -59,19 +59,21 @@ class GatedFfn:
                 needs.append(TensorNeed(name, (size,)))
         return needs
 
-    def forward(self, x: torch.Tensor, step) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, step, slices_ok: bool = True, tag: str = "ffn") -> torch.Tensor:
+        """``slices_ok`` False: the result is wanted as rows of the activations' type (a caller that is no
+        block and adds something to it); ``tag`` keeps the buffers of two feed-forwards of one layer apart."""
         ff = self.spec.intermediate
         n = x.shape[0]
-        act = self.env.workspace.get("ffn_act", n, ff, x.dtype)
+        act = self.env.workspace.get(tag + "_act", n, ff, x.dtype)
         if not self.gate_up.forward_geglu(x, act):
-            gu = self.gate_up.forward(x, tag="gate_up")
+            gu = self.gate_up.forward(x, tag="gate_up" if tag == "ffn" else tag + "_gate_up")
             kernels.gated_act(gu[:, :ff], gu[:, ff:], act, self.spec.activation)
-        return self.down.forward(act, tag="ffn_down", slices_ok=True)    # the block adds it to the residual stream
+        return self.down.forward(act, tag=tag + "_down", slices_ok=slices_ok)    # the block adds it to the residual stream
 
 
 class DenseFfn:
     """``W_down act(W_up x)`` without a gate.  The activation is the spec's, one of
-    ``agave_amd.ops.kernels.UNARY_ACTIVATIONS``.  ``xielu`` has two learned numbers p and q in a tensor
+    ``agave_amd.ops.kernels.UNARY_ACTIVATIONS``.  ``relu2`` is the square of ReLU; ``xielu`` has two learned numbers p and q in a tensor
     of its own:  z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2;
     the two factors are made once at load."""
     prompt_steps_can_be_recorded = True

@@ -52,6 +52,8 @@ def add_branch(h: torch.Tensor, pending: Pending) -> None:
         kernels.residual_norm(h, branch, None, 0.0, None, None, 0.0, src=base)
     elif isinstance(post, RmsNorm):
         kernels.residual_norm(h, branch, post.gain, post.eps, None, None, 0.0, src=base)
+    elif isinstance(post, LayerNorm):
+        kernels.residual_layernorm(h, branch, post.weight, post.bias, post.eps, None, None, None, 0.0, src=base)
     else:
         if base is not None:
             h.copy_(base)
@@ -174,4 +176,61 @@ class RmsNorm(Norm):
                               src=base)
 
 
+class LayerNorm(Norm):
+    """``y = (x - mean(x)) / sqrt(var(x) + eps) * w + b`` with the variance the mean of the squared
+    deviations.  A vector ``scale_by`` and a number ``mult`` that multiply the result (a layer scale and a
+    multiplier on a residual branch) are folded into weight and bias once at load, in 32-bit.  One kernel
+    adds a pending branch through the layer norm after its sublayer and computes this norm."""
+
+    def __init__(self, spec: NormSpec, weights, env: BuildEnv):
+        w = weights.get(spec.weight).to(torch.float32)
+        b = weights.get(spec.bias).to(torch.float32) if spec.bias else None
+        if spec.add_one:
+            w = w + 1.0
+        if spec.scale_by:
+            by = weights.get(spec.scale_by).to(torch.float32)
+            w = w * by
+            b = b * by if b is not None else None
+        if spec.mult != 1.0:
+            w = w * float(spec.mult)
+            b = b * float(spec.mult) if b is not None else None
+        self.weight = w.contiguous().to(env.device)
+        self.bias = b.contiguous().to(env.device) if b is not None else None
+        self.eps = float(spec.eps)
+        self.size = spec.size
+
+    @staticmethod
+    def tensor_needs(spec: NormSpec) -> List[TensorNeed]:
+        needs = [TensorNeed(spec.weight, (spec.size,))]
+        if spec.bias:
+            needs.append(TensorNeed(spec.bias, (spec.size,)))
+        if spec.scale_by:
+            needs.append(TensorNeed(spec.scale_by, (spec.size,)))
+        return needs
+
+    def apply(self, x, out, rows=None) -> None:
+        kernels.residual_layernorm(x, None, None, None, 0.0, out, self.weight, self.bias, self.eps, rows)
+
+    def add_to(self, h, branch) -> None:
+        kernels.residual_layernorm(h, branch, self.weight, self.bias, self.eps, None, None, None, 0.0)
+
+    def add_and_norm(self, h, pending, out, rows=None) -> None:
+        branch, post, base = unpack_pending(pending)
+        if branch is not None and post is not None and not isinstance(post, LayerNorm):
+            add_branch(h, (branch, post, base))     # another kind of norm after the sublayer: its own kernel
+            branch = post = base = None
+        if rows is not None and (branch is not None or base is not None):
+            add_branch(h, (branch, post, base))     # the fused kernel gathers rows only without a branch
+            branch = post = base = None
+        if branch is None and out is None:
+            add_branch(h, (None, None, base))
+            return
+        with_post = branch is not None and post is not None
+        kernels.residual_layernorm(h, branch, post.weight if with_post else None, post.bias if with_post else None,
+                                   post.eps if with_post else 0.0, out, self.weight if out is not None else None,
+                                   self.bias if out is not None else None, self.eps if out is not None else 0.0, rows,
+                                   src=base)
+
+
 register("norm", "rmsnorm", RmsNorm)
+register("norm", "layernorm", LayerNorm)

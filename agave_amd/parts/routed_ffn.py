@@ -1,0 +1,96 @@
+"""A routed feed-forward: a mixture of gated experts with a shared expert.
+
+The router's logits are a 32-bit product of the feed-forward's input with the router matrix (kept in
+32-bit).  Scores are the softmax over all router outputs; the choice goes by score + correction among the
+outputs of the best groups, the weights are the plain scores times a factor (see
+``agave_amd.config.spec.RoutedFfnSpec``).  Outputs past the experts with weights are identity experts:
+their result is the input row.  The chosen experts' rows are summed with their weights, the shared
+expert's row is added.
+
+Nothing on the host depends on the choice: every launch has the same shape whatever the tokens are, so a
+decode step is recorded into a graph like any other.
+"""
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from ..config.spec import RoutedFfnSpec
+from ..ops import kernels, routed
+from ..weights.loader import TensorNeed
+from .base import BuildEnv, register
+from .ffn import GatedFfn
+
+
+class RoutedFfn:
+    @staticmethod
+    def kernel_libraries(spec, dtype):
+        return ("routed_ffn",)
+
+    def __init__(self, spec: RoutedFfnSpec, weights, env: BuildEnv):
+        s = spec
+        if s.activation not in kernels.GATE_ACTIVATIONS:
+            raise ValueError(f"routed feed-forward: unsupported activation {s.activation!r}; known: {sorted(kernels.GATE_ACTIVATIONS)}")
+        self.n_outputs = s.n_experts + s.n_identity
+        if self.n_outputs < 1 or self.n_outputs > routed.MAX_OUTPUTS:
+            raise ValueError(f"routed feed-forward: {self.n_outputs} router outputs (1 to {routed.MAX_OUTPUTS})")
+        if s.groups < 1 or s.groups > 64 or self.n_outputs % s.groups:
+            raise ValueError(f"routed feed-forward: {self.n_outputs} router outputs do not form {s.groups} equal groups (at most 64)")
+        if not 1 <= s.keep_groups <= s.groups:
+            raise ValueError(f"routed feed-forward: {s.keep_groups} of {s.groups} groups kept")
+        if not 1 <= s.top <= s.keep_groups * (self.n_outputs // s.groups):
+            raise ValueError(f"routed feed-forward: {s.top} experts chosen of {s.keep_groups * (self.n_outputs // s.groups)} that can be")
+        self.spec, self.env = spec, env
+        self.act = kernels.GATE_ACTIVATIONS[s.activation]
+        dev = env.device
+        # the router stays 32-bit in both engines
+        self.router = weights.get(s.router).to(torch.float32).contiguous().to(dev)
+        self.correction = weights.get(s.correction).to(torch.float32).contiguous().to(dev) if s.correction else None
+
+        def stack(which: str) -> torch.Tensor:
+            mats = [weights.get(f"{s.expert_prefix}{i}.{which}") for i in range(s.n_experts)]
+            return torch.stack([m.to(env.dtype) for m in mats]).contiguous().to(dev)     # [experts, out, in]
+        if s.n_experts:
+            self.w_gate, self.w_up, self.w_down = stack(s.gate_name), stack(s.up_name), stack(s.down_name)
+        else:
+            self.w_gate = self.w_up = self.w_down = None
+        self.shared = GatedFfn(s.shared, weights, env) if s.shared is not None else None
+
+    @staticmethod
+    def tensor_needs(spec: RoutedFfnSpec) -> List[TensorNeed]:
+        s = spec
+        r = s.n_experts + s.n_identity
+        needs = []
+        for i in range(s.n_experts):
+            p = f"{s.expert_prefix}{i}."
+            needs += [TensorNeed(p + s.gate_name, (s.intermediate, s.hidden)), TensorNeed(p + s.up_name, (s.intermediate, s.hidden)),
+                      TensorNeed(p + s.down_name, (s.hidden, s.intermediate))]
+        needs.append(TensorNeed(s.router, (r, s.hidden)))
+        if s.correction:
+            needs.append(TensorNeed(s.correction, (r,)))
+        if s.shared is not None:
+            needs += GatedFfn.tensor_needs(s.shared)
+        return needs
+
+    def forward(self, x: torch.Tensor, step) -> torch.Tensor:
+        s, ws = self.spec, self.env.workspace
+        n, r, top = x.shape[0], self.n_outputs, s.top
+        logits = ws.get("router_logits", n, r, torch.float32)
+        kernels.gemm_plain(x, self.router, logits)
+        scratch = ws.get("router_scores", n, r, torch.float32)
+        choice = ws.get("router_choice", n, top, torch.int32)
+        weight = ws.get("router_weight", n, top, torch.float32)
+        routed.route_topk(logits, self.correction, scratch, s.groups, s.keep_groups, top, s.route_scale, choice, weight)
+        y = None
+        if s.n_experts:
+            act_rows = ws.get("expert_act", n * top, s.intermediate, x.dtype)
+            y = ws.get("expert_rows", n * top, s.hidden, torch.float32)
+            routed.experts_plain(x, choice.view(-1), self.w_gate, self.w_up, self.w_down, act_rows, y, top, self.act)
+        shared = self.shared.forward(x, step, slices_ok=False, tag="shared_ffn") if self.shared is not None else None
+        out = ws.get("routed_out", n, s.hidden, x.dtype)
+        routed.combine(y, None, choice.view(-1), weight.view(-1), x, shared, out, top, s.n_experts)
+        return out
+
+
+register("ffn", "routed", RoutedFfn)
