@@ -74,7 +74,7 @@ class KVCache:
         # bfloat16 groups whose head size is a multiple of 16 (up to 256) keep their pages in the
         # matrix cores' tile order; the others row by row
         for k in self.group_keys:
-            if k.layout not in ("tiles", "rows"):
+            if k.layout not in ("tiles", "rows", "rows_vt"):
                 raise CacheError(f"unknown page layout {k.layout!r}")
             if k.layout == "tiles" and k.v_head_dim not in (None, k.head_dim):
                 raise CacheError("pages in tile order hold keys and values of one size; a mixer with narrower "
@@ -91,6 +91,10 @@ class KVCache:
                 vd = key.v_head_dim or key.head_dim
                 self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, key.head_dim), dtype=dtype, device=device))
                 self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, vd), dtype=dtype, device=device))
+            elif key.layout == "rows_vt":
+                vd = key.v_head_dim or key.head_dim
+                self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, key.head_dim), dtype=dtype, device=device))
+                self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, vd, PAGE), dtype=dtype, device=device))
             else:
                 self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, hd_k), dtype=dtype, device=device))
                 self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, key.head_dim, PAGE), dtype=dtype, device=device))

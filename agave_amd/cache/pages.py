@@ -105,7 +105,8 @@ class GroupKey:
     v_head_dim: Optional[int] = None   # size of a value head if it differs from the keys'
     # "tiles": K [page, kv head, 64, head_dim] and V transposed [page, kv head, head_dim, 64], in the
     # matrix cores' operand order where the sizes allow; "rows": K and V row by row,
-    # [page, kv head, 64, head_dim] and [page, kv head, 64, v_head_dim], never reordered
+    # [page, kv head, 64, head_dim] and [page, kv head, 64, v_head_dim], never reordered; "rows_vt": K row by
+    # row and V transposed inside a page, [page, kv head, v_head_dim, 64] (a value column's 64 positions in a row)
     layout: str = "tiles"
     # The first positions of a sequence that stay visible whatever the window: the pages that hold them
     # are never given back, and stand in the first columns of a step's table row (``kept_pages``).

@@ -10,7 +10,7 @@
 //   * a gate on the output rows: out *= sigmoid(gate), element by element.
 // Scores, bias, softmax and the sums over values are 32-bit in every element type.
 //
-// Cache pages: K [page][kv head][64 rows][hd]; V [page][kv head][64 rows][vd].
+// Cache pages: K [page][kv head][64 rows][hd]; V transposed [page][kv head][vd][64 rows].
 // Position j of sequence b lies in row j % 64 of the page in column col(j / 64) of table[b]:
 //   col(i) = i < head ? i : head + i - base[b]        (base[b] >= head)
 // so the first `head` columns are the pages that hold the kept first positions, and the
@@ -44,7 +44,7 @@ __global__ void kv_append_rows_kernel(const T* __restrict__ k, long ldk, const T
     }
     for (int i = threadIdx.x; i < nkv * vd; i += blockDim.x) {
         const int g = i / vd, d = i % vd;
-        v_pages[(((size_t)pg * nkv + g) * AGAVE_PAGE + row) * vd + d] = v[(size_t)t * ldv + i];
+        v_pages[(((size_t)pg * nkv + g) * vd + d) * AGAVE_PAGE + row] = v[(size_t)t * ldv + i];
     }
 }
 
@@ -171,10 +171,10 @@ __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
                     for (int pi = 0; pi < BCHUNK / AGAVE_PAGE; ++pi) {
                         const long vp = page_of[pi];
                         if (vp < 0) continue;
-                        const T* vr = v_pages + ((size_t)vp * nkv + kvh) * AGAVE_PAGE * vd + d;
+                        const T* vr = v_pages + (((size_t)vp * nkv + kvh) * vd + d) * AGAVE_PAGE;
                         for (int r = 0; r < AGAVE_PAGE; ++r) {
                             const float w = sc[pi * AGAVE_PAGE + r];
-                            if (w != 0.f) sum = fmaf(w, ld(vr + (size_t)r * vd), sum);   // rows out of range hold w == 0
+                            if (w != 0.f) sum = fmaf(w, ld(vr + r), sum);   // rows out of range hold w == 0
                         }
                     }
                     acc[a] = acc[a] * alpha + sum;
@@ -231,5 +231,302 @@ extern "C" int agave_attn_biased_plain(int dtype, const void* q, long ldq, void*
     else
         AGAVE_CHECK(false, "attn_biased: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("attn_biased_plain");
+    return 0;
+}
+
+// ------------------------------------------------------------------ matrix-core kernel (bfloat16)
+// A wave owns 16 "columns": in a step of many rows, 16 query rows of one head; in a step of one row
+// a sequence, the row's query heads of one key head (the heads of a group read the same keys).  Per
+// page of 64 keys it computes the transposed scores S^T = K Q^T (keys x columns) with
+// v_mfma_f32_16x16x32_bf16, so that a lane holds scores of one column only: the column's running
+// maximum, sum and rescaling factor are the lane's own (and its three partners' in the other lane
+// groups), and the probabilities go from the score registers straight into the B operand of
+// O^T += V^T P^T, whose keys are taken in the order the score registers hold them (the A operand,
+// a value column's keys from the transposed page, is read in that order: two 8-byte loads).
+//   S^T tile of key block kb: lane l holds keys 16 kb + 4 (l / 16) + e, e = 0..3, of column l % 16
+//   O^T block nb:             lane l holds value columns 16 nb + 4 (l / 16) + e of column l % 16
+// Many rows: a workgroup is four waves with 16 rows each, all pages each.  One row: the four waves
+// share the pages of one (row, key head) and wave 0 merges their partial results through LDS.
+// KS = ceil(hd / 32) steps along the head, VB = blocks of 16 value columns (sizes are padded with
+// zeros in registers, never in memory).
+struct MfmaMode {
+    int one_row;                 // 1: a step of one row a sequence
+    const int* cu;               // [sequences + 1] first row of every sequence (many rows)
+    int table_in_lds;            // the bias table's row of this head is copied to LDS (many rows)
+};
+
+template <int KS, int VB>
+__global__ __launch_bounds__(256) void attn_biased_mfma_kernel(BiasedArgs A, MfmaMode M) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int nh = A.nh, nkv = A.nkv, hd = A.hd, vd = A.vd;
+    const int per = nh / nkv;
+
+    // my column: its row, head, position, and whether it exists
+    int row, head, b;
+    bool valid;
+    if (M.one_row) {
+        row = blockIdx.x;
+        b = A.tok_seq[row];
+        const int hg = blockIdx.z * 16 + c;
+        valid = hg < per;
+        head = blockIdx.y * per + (valid ? hg : 0);
+    } else {
+        b = blockIdx.y;
+        const int r0 = M.cu[b] + blockIdx.x * 64, r1 = M.cu[b + 1];
+        if (r0 >= r1) return;                                   // (the whole workgroup: a shorter sequence of the batch)
+        head = blockIdx.z;
+        if (M.table_in_lds) {                                   // (before any wave leaves: all of them meet at the barrier)
+            const float* src = A.bias + (size_t)head * A.bias_len;
+            for (int i = threadIdx.x; i < A.bias_len; i += blockDim.x) lds[i] = src[i];
+            __syncthreads();
+        }
+        row = r0 + w * 16 + c;
+        valid = row < r1;
+        if (r0 + w * 16 >= r1) return;                          // this wave has no rows; no barrier follows in this mode
+        if (!valid) row = r1 - 1;
+    }
+    const int kvh = head / per;
+    const int pos = A.tok_pos[row];
+    // the wave's range of positions (the same in every lane)
+    int pmin = pos, pmax = pos;
+    if (!M.one_row) {
+        pmin = A.tok_pos[M.cu[b] + blockIdx.x * 64 + w * 16];
+        const int last = min(M.cu[b] + blockIdx.x * 64 + w * 16 + 15, M.cu[b + 1] - 1);
+        pmax = A.tok_pos[last];
+    }
+    const int W = A.window, keep = A.keep_first;
+    const int lo = W > 0 ? max(0, pmin - W + 1) : 0;
+    const int first_win = lo / AGAVE_PAGE;
+    const int n_kept = min(first_win, (keep + AGAVE_PAGE - 1) / AGAVE_PAGE);
+    const int n_pg = n_kept + pmax / AGAVE_PAGE - first_win + 1;
+    const int pbase = A.base[b];
+
+    const float* bias_row = nullptr;           // table of my head
+    float slope = 0.f;
+    if (A.bias_mode == 1) slope = A.bias[head];
+    if (A.bias_mode == 2) bias_row = A.bias + (size_t)head * A.bias_len;
+
+    // Q as the B operand: lane holds Q[column c][32 ks + 8 g .. + 8]
+    frag16 qf[KS];
+    const bf16* qrow = (const bf16*)A.q + (size_t)row * A.ldq + (size_t)head * hd;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int k0 = 32 * ks + 8 * g;
+        qf[ks].u = make_uint4(0, 0, 0, 0);
+        if (valid && k0 < hd) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + k0);
+    }
+
+    f32x4_t o[VB];
+#pragma unroll
+    for (int nb = 0; nb < VB; ++nb) o[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    if (A.sink && (!M.one_row || w == 0)) {
+        m = A.sink[head];
+        l = g == 0 ? 1.f : 0.f;                 // the lane groups' sums are added up at the end
+    }
+
+    const int stride = M.one_row ? 4 : 1;
+    for (int idx = M.one_row ? w : 0; idx < n_pg; idx += stride) {
+        const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
+        const int col = page_col(pi, pbase, A.head);
+        long pg = (col >= 0 && col < A.width) ? A.table[(size_t)b * A.width + col] : -1;
+        if (pg < 0 || pg >= A.n_pages) continue;
+        const bf16* kb_ = (const bf16*)A.k_pages + ((size_t)pg * nkv + kvh) * AGAVE_PAGE * hd;
+        const bf16* vb_ = (const bf16*)A.v_pages + ((size_t)pg * nkv + kvh) * (size_t)vd * AGAVE_PAGE;
+        // scores of the page's four key blocks
+        f32x4_t s[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            s[kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const bf16* kr = kb_ + (size_t)(16 * kb + c) * hd + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                frag16 kf;
+                kf.u = make_uint4(0, 0, 0, 0);
+                if (32 * ks + 8 * g < hd) kf.u = *reinterpret_cast<const uint4*>(kr + 32 * ks);
+                s[kb] = mfma_16x16x32(kf, qf[ks], s[kb]);
+            }
+        }
+        // scale, bias, mask; the page's maximum of my column
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int j = pi * AGAVE_PAGE + 16 * kb + 4 * g + e;
+                const int dist = pos - j;
+                const bool see = valid && dist >= 0 && (W == 0 || dist < W || j < keep);
+                float v = s[kb][e] * A.scale;
+                if (A.bias_mode == 1) v -= slope * (float)dist;
+                if (A.bias_mode == 2) {
+                    const int at = see ? (dist < A.bias_len ? dist : A.bias_len - 1) : 0;
+                    v += M.table_in_lds ? lds[at] : bias_row[at];
+                }
+                v = see ? v : -INFINITY;
+                s[kb][e] = v;
+                tile_max = fmaxf(tile_max, v);
+            }
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float m_new = fmaxf(m, tile_max);
+        // (a column that sees nothing of this page and has seen nothing before keeps m = -inf; its p are 0)
+        const float ref = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = m == -INFINITY ? 0.f : __expf(m - ref);
+        float sum = 0.f;
+        frag16 pf[2];
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb) {
+            float p[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                p[e] = __expf(s[kb][e] - ref);          // exp(-inf) = 0 for what is not seen
+                sum += p[e];
+            }
+            const uint32_t lo2 = f32x2_to_bf16x2(p[0], p[1]), hi2 = f32x2_to_bf16x2(p[2], p[3]);
+            if (kb & 1) {
+                pf[kb >> 1].r[2] = lo2;
+                pf[kb >> 1].r[3] = hi2;
+            } else {
+                pf[kb >> 1].r[0] = lo2;
+                pf[kb >> 1].r[1] = hi2;
+            }
+        }
+        l = l * alpha + sum;
+        m = m_new;
+        // O^T = O^T alpha + V^T P^T
+#pragma unroll
+        for (int nb = 0; nb < VB; ++nb) {
+            if (16 * nb < vd) {
+                o[nb] *= alpha;
+                const bf16* vr = vb_ + (size_t)(16 * nb + c) * AGAVE_PAGE + 4 * g;
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    frag16 vf;
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(vr + 32 * h2);
+                    const uint2 a1 = *reinterpret_cast<const uint2*>(vr + 32 * h2 + 16);
+                    vf.u = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                    o[nb] = mfma_16x16x32(vf, pf[h2], o[nb]);
+                }
+            }
+        }
+    }
+    // the column's sum over the four lane groups
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+
+    if (M.one_row) {
+        // waves 1..3 leave (m, l, O^T) in LDS; wave 0 merges
+        const int per_wave = VB * 16 * 16 + 32;
+        if (w > 0) {
+            float* mine = lds + (size_t)(w - 1) * per_wave;
+            if (g == 0) {
+                mine[c] = m;
+                mine[16 + c] = l;
+            }
+#pragma unroll
+            for (int nb = 0; nb < VB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) mine[32 + (16 * nb + 4 * g + e) * 16 + c] = o[nb][e];
+        }
+        __syncthreads();
+        if (w > 0) return;
+        for (int ow = 0; ow < 3; ++ow) {
+            const float* other = lds + (size_t)ow * per_wave;
+            const float m2 = other[c], l2 = other[16 + c];
+            if (m2 == -INFINITY) continue;                      // (per lane: that wave saw nothing for my column)
+            const float m_new = fmaxf(m, m2);
+            const float a1 = m == -INFINITY ? 0.f : __expf(m - m_new), a2 = __expf(m2 - m_new);
+            l = l * a1 + l2 * a2;
+            m = m_new;
+#pragma unroll
+            for (int nb = 0; nb < VB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[nb][e] = o[nb][e] * a1 + other[32 + (16 * nb + 4 * g + e) * 16 + c] * a2;
+        }
+    }
+    if (!valid) return;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    bf16* orow = (bf16*)A.out + (size_t)row * A.ldo + (size_t)head * vd;
+    const bf16* grow = A.gate ? (const bf16*)A.gate + (size_t)row * A.ldg + (size_t)head * vd : nullptr;
+#pragma unroll
+    for (int nb = 0; nb < VB; ++nb) {
+        const int d0 = 16 * nb + 4 * g;
+        if (d0 < vd) {
+            float y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                y[e] = o[nb][e] * inv;
+                if (grow) y[e] *= 1.0f / (1.0f + __expf(-bf16_to_f32(grow[d0 + e])));
+            }
+            uint2 packed;
+            packed.x = f32x2_to_bf16x2(y[0], y[1]);
+            packed.y = f32x2_to_bf16x2(y[2], y[3]);
+            *reinterpret_cast<uint2*>(orow + d0) = packed;
+        }
+    }
+}
+
+template <int KS, int VB>
+static void launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid, size_t lds_bytes, hipStream_t stream) {
+    attn_biased_mfma_kernel<KS, VB><<<grid, 256, lds_bytes, stream>>>(A, M);
+}
+
+#define BIASED_VB(KS_)                                                                                   \
+    switch (vb) {                                                                                        \
+        case 2: launch_biased_mfma<KS_, 2>(A, M, grid, lds_bytes, stream); break;                        \
+        case 4: launch_biased_mfma<KS_, 4>(A, M, grid, lds_bytes, stream); break;                        \
+        case 8: launch_biased_mfma<KS_, 8>(A, M, grid, lds_bytes, stream); break;                        \
+        default: launch_biased_mfma<KS_, 16>(A, M, grid, lds_bytes, stream); break;                      \
+    }
+
+// 1 if the matrix-core kernel takes these sizes (the caller then may call it), else 0
+extern "C" int agave_attn_biased_mfma_ok(int hd, int vd, int ldq, int ldo, int ldg) {
+    return (hd % 8 == 0 && hd <= 256 && vd % 16 == 0 && vd <= 256 && ldq % 8 == 0 && ldo % 4 == 0 && ldg % 4 == 0) ? 1 : 0;
+}
+
+// `cu`: first row of every sequence (device, sequences + 1 entries), used by steps of many rows;
+// `max_rows`: the most rows a sequence brings; `one_row`: every sequence brings one row.
+extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long ldo, const void* gate, long ldg,
+                                      const void* k_pages, const void* v_pages, const int* table, int width, const int* base,
+                                      int head, int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int N,
+                                      int n_seqs, int max_rows, int one_row, int nh, int nkv, int hd, int vd, float scale,
+                                      int window, int keep_first, int bias_mode, const float* bias, int bias_len,
+                                      const float* sink, hipStream_t stream) {
+    BiasedArgs A{q, ldq, out, ldo, gate, ldg, k_pages, v_pages, table, width, base, head, n_pages, tok_seq, tok_pos,
+                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink};
+    if (check_biased(A, N)) return -1;
+    AGAVE_CHECK(agave_attn_biased_mfma_ok(hd, vd, (int)(ldq % 8), (int)(ldo % 4), (int)(ldg % 4)),
+                "attn_biased_mfma: head sizes %d / %d or row strides that the matrix-core kernel does not take", hd, vd);
+    AGAVE_CHECK(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)gate % 8) == 0 && (nh * (long)hd) % 8 == 0,
+                "attn_biased_mfma: rows must be aligned to 16 bytes");
+    AGAVE_CHECK(cu && n_seqs > 0 && max_rows > 0 && (!one_row || N == n_seqs), "attn_biased_mfma: bad step");
+    if (N == 0) return 0;
+    const int ks = hd <= 32 ? 1 : hd <= 64 ? 2 : hd <= 128 ? 4 : 8;
+    const int vb = vd <= 32 ? 2 : vd <= 64 ? 4 : vd <= 128 ? 8 : 16;
+    MfmaMode M{one_row, cu, 0};
+    dim3 grid;
+    size_t lds_bytes = 0;
+    if (one_row) {
+        const int per = nh / nkv;
+        grid = dim3(N, nkv, (per + 15) / 16);
+        lds_bytes = (size_t)3 * (vb * 16 * 16 + 32) * sizeof(float);
+    } else {
+        grid = dim3((max_rows + 63) / 64, n_seqs, nh);
+        AGAVE_CHECK(grid.y <= 65535 && grid.z <= 65535, "attn_biased_mfma: too many sequences or heads for the grid");
+        if (bias_mode == 2 && bias_len <= 8192) {
+            M.table_in_lds = 1;
+            lds_bytes = (size_t)bias_len * sizeof(float);
+        }
+    }
+    switch (ks) {
+        case 1: BIASED_VB(1); break;
+        case 2: BIASED_VB(2); break;
+        case 4: BIASED_VB(4); break;
+        default: BIASED_VB(8); break;
+    }
+    AGAVE_LAUNCH_CHECK("attn_biased_mfma");
     return 0;
 }

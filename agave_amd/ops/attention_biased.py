@@ -21,6 +21,9 @@ kernels.register_signatures(LIBRARY, {
     "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P],
     "agave_attn_biased_plain": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F,
                                 _I, _I, _I, _P, _I, _P, _P],
+    "agave_attn_biased_mfma_ok": [_I, _I, _I, _I, _I],
+    "agave_attn_biased_mfma": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
+                               _F, _I, _I, _I, _P, _I, _P, _P],
 })
 
 
@@ -31,8 +34,8 @@ def _lib():
 def _check_row_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, vd: int, dtype: torch.dtype) -> int:
     if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd) or not k_pages.is_contiguous():
         raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd}], got {tuple(k_pages.shape)}")
-    if v_pages.dim() != 4 or tuple(v_pages.shape[1:]) != (nkv, 64, vd) or not v_pages.is_contiguous():
-        raise ValueError(f"V pages must be contiguous [pages, {nkv}, 64, {vd}], got {tuple(v_pages.shape)}")
+    if v_pages.dim() != 4 or tuple(v_pages.shape[1:]) != (nkv, vd, 64) or not v_pages.is_contiguous():
+        raise ValueError(f"V pages must be contiguous [pages, {nkv}, {vd}, 64], got {tuple(v_pages.shape)}")
     if k_pages.shape[0] != v_pages.shape[0] or k_pages.dtype != dtype or v_pages.dtype != dtype:
         raise ValueError("K and V pages must agree in page count and dtype with the activations")
     return k_pages.shape[0]
@@ -63,12 +66,13 @@ def kv_append_rows(k: torch.Tensor, v: torch.Tensor, k_pages: torch.Tensor, v_pa
 def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torch.Tensor,
               v_pages: torch.Tensor, table: torch.Tensor, base: torch.Tensor, head: int, step, n_heads: int, n_kv: int,
               head_dim: int, v_head_dim: int, scale: float, window: Optional[int], keep_first: int, bias_mode: int,
-              bias: Optional[torch.Tensor], sink: Optional[torch.Tensor]) -> None:
+              bias: Optional[torch.Tensor], sink: Optional[torch.Tensor], force_plain: bool = False) -> None:
     """out[t, h] = sum_j w_j v_j with w = softmax_j(scale q.k_j + bias(h, p - j)) over the keys that token t at
     position p sees (j <= p and (p - j < window or j < keep_first)), the sink's exp(sink_h) added to the
     denominator, times sigmoid(gate[t, h]) element by element.  ``bias``: slopes [heads] (``BIAS_SLOPES``:
     the bias is -slope_h (p - j)) or a table [heads, distances] (``BIAS_TABLE``: distances beyond the table take
-    its last column)."""
+    its last column).  bfloat16 rows with a key size that is a multiple of 8 and a value size that is a multiple of 16
+    (both up to 256) run on the matrix cores, everything else (and everything with ``force_plain``) on the plain kernel."""
     _dev(q, out, gate, k_pages, v_pages, table, base, bias, sink)
     n = step.n_tokens
     ldq, ldo = _rows(q, "q"), _rows(out, "out")
@@ -91,6 +95,18 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
     elif bias_mode != BIAS_NONE:
         raise ValueError(f"attention: unknown bias mode {bias_mode}")
     _f32vec(sink, "sink", n_heads)
+    if q.dtype == torch.bfloat16 and not force_plain and _lib().agave_attn_biased_mfma_ok(head_dim, v_head_dim, ldq, ldo, ldg) \
+            and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0:
+        # the matrix cores: 16 rows of a head a wave in a step of many rows, a row's heads of one key head in a
+        # step of one row a sequence
+        _i32(step.cu_dev, "cu", step.n_seqs + 1)
+        max_rows = max(b - a for a, b in zip(step.cu[:-1], step.cu[1:]))
+        one_row = 1 if (step.is_decode and step.n_tokens == step.n_seqs) else 0
+        library.call(_lib(), "agave_attn_biased_mfma", ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages), ptr(v_pages),
+                     ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), ptr(step.cu_dev), n,
+                     step.n_seqs, max_rows, one_row, n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0),
+                     int(keep_first), bias_mode, ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), stream())
+        return
     library.call(_lib(), "agave_attn_biased_plain", dt(q), ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages),
                  ptr(v_pages), ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n,
                  n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0), int(keep_first), bias_mode,

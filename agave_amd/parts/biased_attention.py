@@ -116,7 +116,7 @@ class BiasedAttention:
 
     def kv_need(self) -> Optional[GroupKey]:
         s = self.spec
-        return GroupKey(s.window, s.n_kv_heads, s.head_dim, v_head_dim=s.v_head_dim, layout="rows",
+        return GroupKey(s.window, s.n_kv_heads, s.head_dim, v_head_dim=s.v_head_dim, layout="rows_vt",
                         keep_first=s.keep_first if s.window is not None else 0)
 
     def state_need(self) -> Optional[StateNeed]:

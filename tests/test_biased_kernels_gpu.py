@@ -40,6 +40,7 @@ class Case:
         from agave_amd.parts.biased_attention import distance_table
         g = torch.Generator().manual_seed(seed)
         self.H, self.G, self.d, self.vd, self.window, self.keep, self.T = H, G, d, vd, window, keep, T
+        self.force_plain = False            # bfloat16 shapes that the matrix-core kernel takes run on the plain one instead
         self.q = torch.randn(T, H, d, generator=g)
         self.k = torch.randn(T, G, d, generator=g)
         self.v = torch.randn(T, G, vd, generator=g)
@@ -77,7 +78,7 @@ class Case:
 
     def key(self):
         from agave_amd.cache import GroupKey
-        return GroupKey(self.window, self.G, self.d, v_head_dim=self.vd, layout="rows",
+        return GroupKey(self.window, self.G, self.d, v_head_dim=self.vd, layout="rows_vt",
                         keep_first=self.keep if self.window is not None else 0)
 
     def run(self, ranges, dtype=torch.float32, cache=None, planner=None, slot=None, pages=40):
@@ -100,7 +101,8 @@ class Case:
             A.kv_append_rows(dev(self.k), dev(self.v), kp, vp, table, base, head, step, self.G, self.d, self.vd)
             out = torch.empty(hi - lo, self.H * self.vd, dtype=dtype, device=DEV)
             A.attention(dev(self.q), out, dev(self.gate) if self.gate is not None else None, kp, vp, table, base, head, step,
-                        self.H, self.G, self.d, self.vd, self.scale, self.window, self.keep, self.mode, self.bias, sink)
+                        self.H, self.G, self.d, self.vd, self.scale, self.window, self.keep, self.mode, self.bias, sink,
+                        force_plain=self.force_plain)
             planner.commit(step)
             got[lo:hi] = out.float().cpu()
         if own:
@@ -123,6 +125,10 @@ SHAPES = [
     (3, 1, 64, 64, 130, 70, "table", False, False),       # one key head, two kept pages
     (2, 2, 8, 40, 64, 64, "none", False, False),          # no bias; window and kept positions of a page each
     (5, 5, 32, 16, 1, 3, "none", True, True),             # a window of the token itself
+    (8, 2, 128, 128, 200, 3, "table", True, True),        # the sizes of large models: the matrix cores in bfloat16
+    (4, 1, 96, 48, 100, 0, "slopes", True, False),        # sizes that fill the matrix cores' steps only in part
+    (34, 1, 32, 32, None, 0, "table", False, True),       # more heads to a key head than a wave has columns
+    (2, 2, 256, 256, 64, 64, "slopes", False, False),     # the largest heads
 ]
 
 
@@ -135,6 +141,9 @@ def test_attention_whole_in_pieces_and_token_by_token(shape, dtype):
     ref = c.plain()
     for first, piece in ((T, 1), (200, 1), (1, 1), (3, 2), (50, 37), (64, 64)):
         close(c.run(cuts(T, first, piece), dtype), ref, dtype, f"{shape} first {first} pieces of {piece}")
+    if dtype == torch.bfloat16:
+        c.force_plain = True
+        close(c.run(cuts(T, 180, 1), dtype), ref, dtype, f"{shape} on the plain kernel")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -199,7 +208,9 @@ def test_a_dominant_key_just_inside_and_just_outside(window, keep, dtype):
     T = 420
     for j0, inside_until in ([(150, 150 + window - 1)] + ([(keep - 1, T - 1), (keep, keep + window - 1)] if keep else [])):
         # (a slope on the distance would bury a key hundreds of positions back: the table's bias is bounded)
-        c = Case(4, 2, 16, 8, window, keep, "slopes" if window == 48 else "table", True, False, T=T, seed=j0)
+        # (values of 16 in bfloat16: the matrix-core kernel; of 8: the plain one)
+        c = Case(4, 2, 16, 16 if (dtype == torch.bfloat16 and window != 100) else 8, window, keep,
+                 "slopes" if window == 48 else "table", True, False, T=T, seed=j0)
         one_key_stands_out(c, j0, 5.0)
         c.rounded(dtype)
         ref = c.plain()

@@ -86,7 +86,7 @@ def test_buckets_of_distances():
 
 
 def test_first_pages_are_kept_and_stand_first_in_the_table():
-    key = GroupKey(100, 2, 16, v_head_dim=8, layout="rows", keep_first=70)        # two kept pages
+    key = GroupKey(100, 2, 16, v_head_dim=8, layout="rows_vt", keep_first=70)        # two kept pages
     assert key.kept_pages == 2 and GroupKey(None, 2, 16, keep_first=70).kept_pages == 0
     g = GroupPages(key, 12, 2)
     base, pages = g.plan(0, 0, 50)
@@ -108,17 +108,17 @@ def test_first_pages_are_kept_and_stand_first_in_the_table():
     g.release(0)
     assert g.pool.n_free == 12
     # the window still overlaps the kept pages: the columns are the pages in order
-    g2 = GroupPages(GroupKey(100, 1, 8, layout="rows", keep_first=10), 8, 1)
+    g2 = GroupPages(GroupKey(100, 1, 8, layout="rows_vt", keep_first=10), 8, 1)
     base, pages = g2.plan(0, 0, 130)
     assert base == 1 and len(pages) == 3
 
 
 def test_readers_with_different_windows_share_the_wider_need():
-    a = GroupKey(72, 2, 8, v_head_dim=4, layout="rows")
-    b = GroupKey(200, 2, 8, v_head_dim=4, layout="rows", keep_first=3)
+    a = GroupKey(72, 2, 8, v_head_dim=4, layout="rows_vt")
+    b = GroupKey(200, 2, 8, v_head_dim=4, layout="rows_vt", keep_first=3)
     both = a.covering(b)
-    assert both.window == 200 and both.keep_first == 3 and a.covering(GroupKey(None, 2, 8, v_head_dim=4, layout="rows")).window is None
-    assert a.covering(GroupKey(72, 2, 16, v_head_dim=4, layout="rows")) is None
+    assert both.window == 200 and both.keep_first == 3 and a.covering(GroupKey(None, 2, 8, v_head_dim=4, layout="rows_vt")).window is None
+    assert a.covering(GroupKey(72, 2, 16, v_head_dim=4, layout="rows_vt")) is None
     cache = KVCache({0: both}, {}, 2, {both: 10}, torch.float32, None, 1024)
     s = cache.alloc_slot()
     cache.check_pieces([s], [[300], [300]])

@@ -132,7 +132,7 @@ def test_the_cache_as_the_mixers_asked(models):
     assert set(eng.cache.group_of_memory) == {0, 1, 3}            # layers 2 and 4 read layer 1's memory
     by_mem = {m: eng.cache.group_keys[g] for m, g in eng.cache.group_of_memory.items()}
     assert by_mem[1].window == 90 and by_mem[0].keep_first == 5 and by_mem[3].kept_pages == 2      # the widest reader's window
-    assert all(k.layout == "rows" for k in keys) and by_mem[1].v_head_dim == 8
+    assert all(k.layout == "rows_vt" for k in keys) and by_mem[1].v_head_dim == 8
     from agave_amd.ops import library
     slot = eng.alloc_slot()
     eng.step([slot], [[1, 2]])
