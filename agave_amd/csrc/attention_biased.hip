@@ -235,46 +235,60 @@ extern "C" int agave_attn_biased_plain(int dtype, const void* q, long ldq, void*
 }
 
 // ------------------------------------------------------------------ matrix-core kernel (bfloat16)
-// A wave owns 16 "columns": in a step of many rows, 16 query rows of one head; in a step of one row
-// a sequence, the row's query heads of one key head (the heads of a group read the same keys).  Per
+// A wave owns NC blocks of 16 "columns": in a step of many rows, 16 NC query rows of one head; in a step of
+// one row a sequence, the row's query heads of one key head (the heads of a group read the same keys).  Per
 // page of 64 keys it computes the transposed scores S^T = K Q^T (keys x columns) with
-// v_mfma_f32_16x16x32_bf16, so that a lane holds scores of one column only: the column's running
+// v_mfma_f32_16x16x32_bf16, so that a lane holds scores of one column a block only: the column's running
 // maximum, sum and rescaling factor are the lane's own (and its three partners' in the other lane
 // groups), and the probabilities go from the score registers straight into the B operand of
 // O^T += V^T P^T, whose keys are taken in the order the score registers hold them (the A operand,
-// a value column's keys from the transposed page, is read in that order: two 8-byte loads).
+// a value column's keys from the transposed page, is read in that order: two 8-byte loads).  A key or
+// value operand that was loaded serves all NC column blocks.
 //   S^T tile of key block kb: lane l holds keys 16 kb + 4 (l / 16) + e, e = 0..3, of column l % 16
 //   O^T block nb:             lane l holds value columns 16 nb + 4 (l / 16) + e of column l % 16
-// Many rows: a workgroup is four waves with 16 rows each, all pages each.  One row: the four waves
-// share the pages of one (row, key head) and wave 0 merges their partial results through LDS.
-// KS = ceil(hd / 32) steps along the head, VB = blocks of 16 value columns (sizes are padded with
-// zeros in registers, never in memory).
+// Many rows: a workgroup is four waves with 16 NC rows each, all pages each.  One row: the workgroup's
+// waves (four or eight) share the pages of one (row, key head) and wave 0 merges their partial results
+// through LDS.  KS = ceil(hd / 32) steps along the head, VB = blocks of 16 value columns (sizes are
+// padded with zeros in registers, never in memory).
 struct MfmaMode {
     int one_row;                 // 1: a step of one row a sequence
     const int* cu;               // [sequences + 1] first row of every sequence (many rows)
     int table_in_lds;            // the bias table's row of this head is copied to LDS (many rows)
 };
 
-template <int KS, int VB>
-__global__ __launch_bounds__(256) void attn_biased_mfma_kernel(BiasedArgs A, MfmaMode M) {
-    extern __shared__ float lds[];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+template <int KS, int VB, int NC>
+__global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, MfmaMode M) {
+    extern __shared__ float lds_generic[];
+    // (every LDS access goes through a pointer that says so: no pointer may end up chosen between the two memories)
+    typedef __attribute__((address_space(3))) float lds_float;
+    lds_float* lds = (lds_float*)lds_generic;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int nh = A.nh, nkv = A.nkv, hd = A.hd, vd = A.vd;
     const int per = nh / nkv;
+    constexpr int WROWS = 16 * NC;                  // rows a wave in a step of many rows
 
-    // my column: its row, head, position, and whether it exists
-    int row, head, b;
-    bool valid;
+    // my columns (one a block): row, position, whether it exists; the head is the same for all in a step of many rows
+    int row[NC], pos[NC], head, b;
+    bool valid[NC];
+    int pmin, pmax;                                 // the wave's range of positions (the same in every lane)
     if (M.one_row) {
-        row = blockIdx.x;
-        b = A.tok_seq[row];
+        row[0] = blockIdx.x;
+        b = A.tok_seq[row[0]];
         const int hg = blockIdx.z * 16 + c;
-        valid = hg < per;
-        head = blockIdx.y * per + (valid ? hg : 0);
+        valid[0] = hg < per;
+        head = blockIdx.y * per + (valid[0] ? hg : 0);
+        pos[0] = A.tok_pos[row[0]];
+        pmin = pmax = pos[0];
+#pragma unroll
+        for (int cb = 1; cb < NC; ++cb) {           // (one block of columns in this mode)
+            row[cb] = row[0];
+            pos[cb] = pos[0];
+            valid[cb] = false;
+        }
     } else {
         b = blockIdx.y;
-        const int r0 = M.cu[b] + blockIdx.x * 64, r1 = M.cu[b + 1];
+        const int r0 = M.cu[b] + blockIdx.x * 4 * WROWS, r1 = M.cu[b + 1];
         if (r0 >= r1) return;                                   // (the whole workgroup: a shorter sequence of the batch)
         head = blockIdx.z;
         if (M.table_in_lds) {                                   // (before any wave leaves: all of them meet at the barrier)
@@ -282,20 +296,19 @@ __global__ __launch_bounds__(256) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
             for (int i = threadIdx.x; i < A.bias_len; i += blockDim.x) lds[i] = src[i];
             __syncthreads();
         }
-        row = r0 + w * 16 + c;
-        valid = row < r1;
-        if (r0 + w * 16 >= r1) return;                          // this wave has no rows; no barrier follows in this mode
-        if (!valid) row = r1 - 1;
+        const int wr0 = r0 + w * WROWS;
+        if (wr0 >= r1) return;                                  // this wave has no rows; no barrier follows in this mode
+#pragma unroll
+        for (int cb = 0; cb < NC; ++cb) {
+            row[cb] = wr0 + 16 * cb + c;
+            valid[cb] = row[cb] < r1;
+            if (!valid[cb]) row[cb] = r1 - 1;
+            pos[cb] = A.tok_pos[row[cb]];
+        }
+        pmin = A.tok_pos[wr0];
+        pmax = A.tok_pos[min(wr0 + WROWS, r1) - 1];
     }
     const int kvh = head / per;
-    const int pos = A.tok_pos[row];
-    // the wave's range of positions (the same in every lane)
-    int pmin = pos, pmax = pos;
-    if (!M.one_row) {
-        pmin = A.tok_pos[M.cu[b] + blockIdx.x * 64 + w * 16];
-        const int last = min(M.cu[b] + blockIdx.x * 64 + w * 16 + 15, M.cu[b + 1] - 1);
-        pmax = A.tok_pos[last];
-    }
     const int W = A.window, keep = A.keep_first;
     const int lo = W > 0 ? max(0, pmin - W + 1) : 0;
     const int first_win = lo / AGAVE_PAGE;
@@ -309,177 +322,257 @@ __global__ __launch_bounds__(256) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
     if (A.bias_mode == 2) bias_row = A.bias + (size_t)head * A.bias_len;
 
     // Q as the B operand: lane holds Q[column c][32 ks + 8 g .. + 8]
-    frag16 qf[KS];
-    const bf16* qrow = (const bf16*)A.q + (size_t)row * A.ldq + (size_t)head * hd;
+    frag16 qf[NC][KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const int k0 = 32 * ks + 8 * g;
-        qf[ks].u = make_uint4(0, 0, 0, 0);
-        if (valid && k0 < hd) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + k0);
+    for (int cb = 0; cb < NC; ++cb) {
+        const bf16* qrow = (const bf16*)A.q + (size_t)row[cb] * A.ldq + (size_t)head * hd;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            // (every load is written without a condition, from an address inside the row, and emptied afterwards
+            // where it lies past the head's end: a load under a per-lane condition is waited for on the spot)
+            const int k0 = 32 * ks + 8 * g;
+            const uint4 got = *reinterpret_cast<const uint4*>(qrow + (k0 < hd ? k0 : 0));
+            qf[cb][ks].u = (valid[cb] && k0 < hd) ? got : make_uint4(0, 0, 0, 0);
+        }
     }
 
-    f32x4_t o[VB];
+    f32x4_t o[NC][VB];
+    float m[NC], l[NC];
 #pragma unroll
-    for (int nb = 0; nb < VB; ++nb) o[nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.f;
-    if (A.sink && (!M.one_row || w == 0)) {
-        m = A.sink[head];
-        l = g == 0 ? 1.f : 0.f;                 // the lane groups' sums are added up at the end
+    for (int cb = 0; cb < NC; ++cb) {
+#pragma unroll
+        for (int nb = 0; nb < VB; ++nb) o[cb][nb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        m[cb] = -INFINITY;
+        l[cb] = 0.f;
+        if (A.sink && (!M.one_row || w == 0)) {
+            m[cb] = A.sink[head];
+            l[cb] = g == 0 ? 1.f : 0.f;         // the lane groups' sums are added up at the end
+        }
     }
 
-    const int stride = M.one_row ? 4 : 1;
-    for (int idx = M.one_row ? w : 0; idx < n_pg; idx += stride) {
+    const int stride = M.one_row ? nw : 1;
+    auto page_of = [&](int idx) -> long {
+        if (idx >= n_pg) return -1;
         const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
         const int col = page_col(pi, pbase, A.head);
-        long pg = (col >= 0 && col < A.width) ? A.table[(size_t)b * A.width + col] : -1;
-        if (pg < 0 || pg >= A.n_pages) continue;
-        const bf16* kb_ = (const bf16*)A.k_pages + ((size_t)pg * nkv + kvh) * AGAVE_PAGE * hd;
-        const bf16* vb_ = (const bf16*)A.v_pages + ((size_t)pg * nkv + kvh) * (size_t)vd * AGAVE_PAGE;
+        const long pg = (col >= 0 && col < A.width) ? A.table[(size_t)b * A.width + col] : -1;
+        return pg < A.n_pages ? pg : -1;
+    };
+    int idx = M.one_row ? w : 0;
+    long pg = page_of(idx);
+    for (; idx < n_pg; idx += stride) {
+        const long pg_next = page_of(idx + stride);         // asked for now, used in the next turn
+        const long pg_now = pg;
+        pg = pg_next;
+        if (pg_now < 0) continue;
+        const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
+        const bf16* kb_ = (const bf16*)A.k_pages + ((size_t)pg_now * nkv + kvh) * AGAVE_PAGE * hd;
+        const bf16* vb_ = (const bf16*)A.v_pages + ((size_t)pg_now * nkv + kvh) * (size_t)vd * AGAVE_PAGE;
+        // What the page needs from memory is asked for before any of it is used (a wave's loads come back in the
+        // order they left): the bias where it is read from memory, the value operands where the registers allow, then
+        // the keys.
+        constexpr bool V_AHEAD = VB <= 8 && NC == 1;
+        float bv[NC][4][4];
+        if (A.bias_mode == 2 && !M.table_in_lds) {
+#pragma unroll
+            for (int cb = 0; cb < NC; ++cb)
+#pragma unroll
+                for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int dist = pos[cb] - (pi * AGAVE_PAGE + 16 * kb + 4 * g + e);
+                        bv[cb][kb][e] = bias_row[dist < 0 ? 0 : (dist < A.bias_len ? dist : A.bias_len - 1)];
+                    }
+        }
+        frag16 va[V_AHEAD ? VB : 1][2];
+        if (V_AHEAD) {
+#pragma unroll
+            for (int nb = 0; nb < VB; ++nb) {
+                // (a block past the value size reads the first block again and is not used)
+                const bf16* vr = vb_ + (size_t)((16 * nb < vd ? 16 * nb : 0) + c) * AGAVE_PAGE + 4 * g;
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const uint2 a0 = *reinterpret_cast<const uint2*>(vr + 32 * h2);
+                    const uint2 a1 = *reinterpret_cast<const uint2*>(vr + 32 * h2 + 16);
+                    va[V_AHEAD ? nb : 0][h2].u = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                }
+            }
+        }
         // scores of the page's four key blocks
-        f32x4_t s[4];
+        f32x4_t s[NC][4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-            s[kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             const bf16* kr = kb_ + (size_t)(16 * kb + c) * hd + 8 * g;
+            frag16 kf[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                frag16 kf;
-                kf.u = make_uint4(0, 0, 0, 0);
-                if (32 * ks + 8 * g < hd) kf.u = *reinterpret_cast<const uint4*>(kr + 32 * ks);
-                s[kb] = mfma_16x16x32(kf, qf[ks], s[kb]);
+                const bool in = 32 * ks + 8 * g < hd;
+                const uint4 got = *reinterpret_cast<const uint4*>(kr + (in ? 32 * ks : -8 * g));
+                kf[ks].u = in ? got : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int cb = 0; cb < NC; ++cb) {
+                s[cb][kb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) s[cb][kb] = mfma_16x16x32(kf[ks], qf[cb][ks], s[cb][kb]);
             }
         }
-        // scale, bias, mask; the page's maximum of my column
-        float tile_max = -INFINITY;
+        // scale, bias, mask, softmax a column block at a time
+        frag16 pf[NC][2];
+        float alpha[NC];
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
+        for (int cb = 0; cb < NC; ++cb) {
+            float tile_max = -INFINITY;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int j = pi * AGAVE_PAGE + 16 * kb + 4 * g + e;
-                const int dist = pos - j;
-                const bool see = valid && dist >= 0 && (W == 0 || dist < W || j < keep);
-                float v = s[kb][e] * A.scale;
-                if (A.bias_mode == 1) v -= slope * (float)dist;
-                if (A.bias_mode == 2) {
-                    const int at = see ? (dist < A.bias_len ? dist : A.bias_len - 1) : 0;
-                    v += M.table_in_lds ? lds[at] : bias_row[at];
+            for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = pi * AGAVE_PAGE + 16 * kb + 4 * g + e;
+                    const int dist = pos[cb] - j;
+                    const bool see = valid[cb] && dist >= 0 && (W == 0 || dist < W || j < keep);
+                    float v = s[cb][kb][e] * A.scale;
+                    if (A.bias_mode == 1) v -= slope * (float)dist;
+                    if (A.bias_mode == 2) {
+                        const int at = see ? (dist < A.bias_len ? dist : A.bias_len - 1) : 0;
+                        v += M.table_in_lds ? lds[at] : bv[cb][kb][e];
+                    }
+                    v = see ? v : -INFINITY;
+                    s[cb][kb][e] = v;
+                    tile_max = fmaxf(tile_max, v);
                 }
-                v = see ? v : -INFINITY;
-                s[kb][e] = v;
-                tile_max = fmaxf(tile_max, v);
             }
-        }
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-        const float m_new = fmaxf(m, tile_max);
-        // (a column that sees nothing of this page and has seen nothing before keeps m = -inf; its p are 0)
-        const float ref = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = m == -INFINITY ? 0.f : __expf(m - ref);
-        float sum = 0.f;
-        frag16 pf[2];
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+            const float m_new = fmaxf(m[cb], tile_max);
+            // (a column that sees nothing of this page and has seen nothing before keeps m = -inf; its p are 0)
+            const float ref = m_new == -INFINITY ? 0.f : m_new;
+            alpha[cb] = m[cb] == -INFINITY ? 0.f : __expf(m[cb] - ref);
+            float sum = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 4; ++kb) {
-            float p[4];
+            for (int kb = 0; kb < 4; ++kb) {
+                float p[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                p[e] = __expf(s[kb][e] - ref);          // exp(-inf) = 0 for what is not seen
-                sum += p[e];
+                for (int e = 0; e < 4; ++e) {
+                    p[e] = __expf(s[cb][kb][e] - ref);          // exp(-inf) = 0 for what is not seen
+                    sum += p[e];
+                }
+                const uint32_t lo2 = f32x2_to_bf16x2(p[0], p[1]), hi2 = f32x2_to_bf16x2(p[2], p[3]);
+                if (kb & 1) {
+                    pf[cb][kb >> 1].r[2] = lo2;
+                    pf[cb][kb >> 1].r[3] = hi2;
+                } else {
+                    pf[cb][kb >> 1].r[0] = lo2;
+                    pf[cb][kb >> 1].r[1] = hi2;
+                }
             }
-            const uint32_t lo2 = f32x2_to_bf16x2(p[0], p[1]), hi2 = f32x2_to_bf16x2(p[2], p[3]);
-            if (kb & 1) {
-                pf[kb >> 1].r[2] = lo2;
-                pf[kb >> 1].r[3] = hi2;
-            } else {
-                pf[kb >> 1].r[0] = lo2;
-                pf[kb >> 1].r[1] = hi2;
-            }
+            l[cb] = l[cb] * alpha[cb] + sum;
+            m[cb] = m_new;
         }
-        l = l * alpha + sum;
-        m = m_new;
         // O^T = O^T alpha + V^T P^T
 #pragma unroll
         for (int nb = 0; nb < VB; ++nb) {
             if (16 * nb < vd) {
-                o[nb] *= alpha;
-                const bf16* vr = vb_ + (size_t)(16 * nb + c) * AGAVE_PAGE + 4 * g;
+                frag16 vf[2];
+                if (V_AHEAD) {
+                    vf[0] = va[V_AHEAD ? nb : 0][0];
+                    vf[1] = va[V_AHEAD ? nb : 0][1];
+                } else {
+                    const bf16* vr = vb_ + (size_t)(16 * nb + c) * AGAVE_PAGE + 4 * g;
 #pragma unroll
-                for (int h2 = 0; h2 < 2; ++h2) {
-                    frag16 vf;
-                    const uint2 a0 = *reinterpret_cast<const uint2*>(vr + 32 * h2);
-                    const uint2 a1 = *reinterpret_cast<const uint2*>(vr + 32 * h2 + 16);
-                    vf.u = make_uint4(a0.x, a0.y, a1.x, a1.y);
-                    o[nb] = mfma_16x16x32(vf, pf[h2], o[nb]);
+                    for (int h2 = 0; h2 < 2; ++h2) {
+                        const uint2 a0 = *reinterpret_cast<const uint2*>(vr + 32 * h2);
+                        const uint2 a1 = *reinterpret_cast<const uint2*>(vr + 32 * h2 + 16);
+                        vf[h2].u = make_uint4(a0.x, a0.y, a1.x, a1.y);
+                    }
+                }
+#pragma unroll
+                for (int cb = 0; cb < NC; ++cb) {
+                    o[cb][nb] *= alpha[cb];
+                    o[cb][nb] = mfma_16x16x32(vf[0], pf[cb][0], o[cb][nb]);
+                    o[cb][nb] = mfma_16x16x32(vf[1], pf[cb][1], o[cb][nb]);
                 }
             }
         }
     }
-    // the column's sum over the four lane groups
-    l += __shfl_xor(l, 16);
-    l += __shfl_xor(l, 32);
+    // the columns' sums over the four lane groups
+#pragma unroll
+    for (int cb = 0; cb < NC; ++cb) {
+        l[cb] += __shfl_xor(l[cb], 16);
+        l[cb] += __shfl_xor(l[cb], 32);
+    }
 
     if (M.one_row) {
-        // waves 1..3 leave (m, l, O^T) in LDS; wave 0 merges
+        // the other waves leave (m, l, O^T) in LDS; wave 0 merges
         const int per_wave = VB * 16 * 16 + 32;
         if (w > 0) {
-            float* mine = lds + (size_t)(w - 1) * per_wave;
+            lds_float* mine = lds + (size_t)(w - 1) * per_wave;
             if (g == 0) {
-                mine[c] = m;
-                mine[16 + c] = l;
+                mine[c] = m[0];
+                mine[16 + c] = l[0];
             }
 #pragma unroll
             for (int nb = 0; nb < VB; ++nb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) mine[32 + (16 * nb + 4 * g + e) * 16 + c] = o[nb][e];
+                for (int e = 0; e < 4; ++e) mine[32 + (16 * nb + 4 * g + e) * 16 + c] = o[0][nb][e];
         }
         __syncthreads();
         if (w > 0) return;
-        for (int ow = 0; ow < 3; ++ow) {
-            const float* other = lds + (size_t)ow * per_wave;
+        for (int ow = 0; ow < nw - 1; ++ow) {
+            const lds_float* other = lds + (size_t)ow * per_wave;
             const float m2 = other[c], l2 = other[16 + c];
             if (m2 == -INFINITY) continue;                      // (per lane: that wave saw nothing for my column)
-            const float m_new = fmaxf(m, m2);
-            const float a1 = m == -INFINITY ? 0.f : __expf(m - m_new), a2 = __expf(m2 - m_new);
-            l = l * a1 + l2 * a2;
-            m = m_new;
+            const float m_new = fmaxf(m[0], m2);
+            const float a1 = m[0] == -INFINITY ? 0.f : __expf(m[0] - m_new), a2 = __expf(m2 - m_new);
+            l[0] = l[0] * a1 + l2 * a2;
+            m[0] = m_new;
 #pragma unroll
             for (int nb = 0; nb < VB; ++nb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[nb][e] = o[nb][e] * a1 + other[32 + (16 * nb + 4 * g + e) * 16 + c] * a2;
+                for (int e = 0; e < 4; ++e) o[0][nb][e] = o[0][nb][e] * a1 + other[32 + (16 * nb + 4 * g + e) * 16 + c] * a2;
         }
     }
-    if (!valid) return;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    bf16* orow = (bf16*)A.out + (size_t)row * A.ldo + (size_t)head * vd;
-    const bf16* grow = A.gate ? (const bf16*)A.gate + (size_t)row * A.ldg + (size_t)head * vd : nullptr;
 #pragma unroll
-    for (int nb = 0; nb < VB; ++nb) {
-        const int d0 = 16 * nb + 4 * g;
-        if (d0 < vd) {
-            float y[4];
+    for (int cb = 0; cb < NC; ++cb) {
+        if (!valid[cb]) continue;
+        const float inv = l[cb] > 0.f ? 1.0f / l[cb] : 0.f;
+        bf16* orow = (bf16*)A.out + (size_t)row[cb] * A.ldo + (size_t)head * vd;
+        const bf16* grow = A.gate ? (const bf16*)A.gate + (size_t)row[cb] * A.ldg + (size_t)head * vd : nullptr;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                y[e] = o[nb][e] * inv;
-                if (grow) y[e] *= 1.0f / (1.0f + __expf(-bf16_to_f32(grow[d0 + e])));
+        for (int nb = 0; nb < VB; ++nb) {
+            const int d0 = 16 * nb + 4 * g;
+            if (d0 < vd) {
+                float y[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    y[e] = o[cb][nb][e] * inv;
+                    if (grow) y[e] *= 1.0f / (1.0f + __expf(-bf16_to_f32(grow[d0 + e])));
+                }
+                uint2 packed;
+                packed.x = f32x2_to_bf16x2(y[0], y[1]);
+                packed.y = f32x2_to_bf16x2(y[2], y[3]);
+                *reinterpret_cast<uint2*>(orow + d0) = packed;
             }
-            uint2 packed;
-            packed.x = f32x2_to_bf16x2(y[0], y[1]);
-            packed.y = f32x2_to_bf16x2(y[2], y[3]);
-            *reinterpret_cast<uint2*>(orow + d0) = packed;
         }
     }
 }
 
 template <int KS, int VB>
-static void launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid, size_t lds_bytes, hipStream_t stream) {
-    attn_biased_mfma_kernel<KS, VB><<<grid, 256, lds_bytes, stream>>>(A, M);
+static void launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid, int threads, int nc, size_t lds_bytes,
+                               hipStream_t stream) {
+    if (nc == 2) {
+        if constexpr (VB <= 8)
+            attn_biased_mfma_kernel<KS, VB, 2><<<grid, threads, lds_bytes, stream>>>(A, M);
+    } else {
+        attn_biased_mfma_kernel<KS, VB, 1><<<grid, threads, lds_bytes, stream>>>(A, M);
+    }
 }
 
 #define BIASED_VB(KS_)                                                                                   \
     switch (vb) {                                                                                        \
-        case 2: launch_biased_mfma<KS_, 2>(A, M, grid, lds_bytes, stream); break;                        \
-        case 4: launch_biased_mfma<KS_, 4>(A, M, grid, lds_bytes, stream); break;                        \
-        case 8: launch_biased_mfma<KS_, 8>(A, M, grid, lds_bytes, stream); break;                        \
-        default: launch_biased_mfma<KS_, 16>(A, M, grid, lds_bytes, stream); break;                      \
+        case 2: launch_biased_mfma<KS_, 2>(A, M, grid, threads, nc, lds_bytes, stream); break;           \
+        case 4: launch_biased_mfma<KS_, 4>(A, M, grid, threads, nc, lds_bytes, stream); break;           \
+        case 8: launch_biased_mfma<KS_, 8>(A, M, grid, threads, nc, lds_bytes, stream); break;           \
+        default: launch_biased_mfma<KS_, 16>(A, M, grid, threads, nc, lds_bytes, stream); break;         \
     }
 
 // 1 if the matrix-core kernel takes these sizes (the caller then may call it), else 0
@@ -509,12 +602,18 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
     MfmaMode M{one_row, cu, 0};
     dim3 grid;
     size_t lds_bytes = 0;
+    int threads = 256, nc = 1;
     if (one_row) {
+        // eight waves share a row's pages where their partial results fit the LDS, else four
         const int per = nh / nkv;
+        const int nw = vb <= 8 ? 8 : 4;
+        threads = 64 * nw;
         grid = dim3(N, nkv, (per + 15) / 16);
-        lds_bytes = (size_t)3 * (vb * 16 * 16 + 32) * sizeof(float);
+        lds_bytes = (size_t)(nw - 1) * (vb * 16 * 16 + 32) * sizeof(float);
     } else {
-        grid = dim3((max_rows + 63) / 64, n_seqs, nh);
+        // 32 rows a wave where the step is long enough to fill the chip that way and the registers allow
+        nc = (vb <= 8 && (long)((max_rows + 127) / 128) * n_seqs * nh >= 256) ? 2 : 1;
+        grid = dim3((max_rows + 64 * nc - 1) / (64 * nc), n_seqs, nh);
         AGAVE_CHECK(grid.y <= 65535 && grid.z <= 65535, "attn_biased_mfma: too many sequences or heads for the grid");
         if (bias_mode == 2 && bias_len <= 8192) {
             M.table_in_lds = 1;

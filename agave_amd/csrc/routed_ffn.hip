@@ -90,6 +90,158 @@ extern "C" int agave_route_topk(const float* z, long ldz, const float* correctio
     return 0;
 }
 
+// ------------------------------------------------------------------ router product and choice in one kernel
+// A workgroup takes ROUTE_ROWS tokens: its waves share the router's outputs (a wave per output in turn, the lanes
+// along the width, a weight row read once for all of the workgroup's tokens), the logits wait in LDS, and one
+// thread per token then chooses as route_topk_kernel does.  The router matrix is 32-bit; the rows may be bfloat16.
+#define ROUTE_ROWS 8
+// eight neighbours along the width as floats (16 bytes of bfloat16, 32 of float)
+__device__ __forceinline__ void load8(const bf16* p, float* v) {
+    const uint4 u = *reinterpret_cast<const uint4*>(p);
+    const uint32_t r[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(r[i] << 16);
+        v[2 * i + 1] = __uint_as_float(r[i] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ void load8(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+// WIDE: the width is a multiple of 8 and the rows are aligned, so a lane takes eight neighbours at a time (a
+// fraction of the loads, many of them in flight); otherwise element by element.  The workgroup's waves (4, or 16
+// where few tokens leave the chip idle) take the outputs in turn.
+template <typename T, bool WIDE>
+__global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ router,
+                                                          const float* __restrict__ correction, int N, int K, int R, int groups,
+                                                          int keep, int top, float scale, int* __restrict__ choice,
+                                                          float* __restrict__ weight) {
+    extern __shared__ float zs[];                      // [ROUTE_ROWS][R]
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int t0 = blockIdx.x * ROUTE_ROWS;
+    const int rows = min(ROUTE_ROWS, N - t0);
+    for (int r = w; r < R; r += nw) {
+        const float* wr = router + (size_t)r * K;
+        float acc[ROUTE_ROWS];
+#pragma unroll
+        for (int i = 0; i < ROUTE_ROWS; ++i) acc[i] = 0.f;
+        if (WIDE) {
+#pragma unroll 2
+            for (int k = 8 * lane; k < K; k += 512) {
+                float wk[8];
+                load8(wr + k, wk);
+#pragma unroll
+                for (int i = 0; i < ROUTE_ROWS; ++i) {
+                    const int t = t0 + (i < rows ? i : 0);
+                    float xv[8];
+                    load8(x + (size_t)t * ldx + k, xv);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[i] = fmaf(xv[j], wk[j], acc[i]);
+                }
+            }
+        } else {
+            for (int k = lane; k < K; k += 64) {
+                const float wk = wr[k];
+#pragma unroll
+                for (int i = 0; i < ROUTE_ROWS; ++i) {
+                    const int t = t0 + (i < rows ? i : 0);
+                    acc[i] = fmaf(ld(x + (size_t)t * ldx + k), wk, acc[i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < ROUTE_ROWS; ++i) {
+            const float sum = wave_sum(acc[i]);
+            if (lane == 0) zs[i * R + r] = sum;
+        }
+    }
+    __syncthreads();
+    const int i = threadIdx.x;
+    if (i >= rows) return;
+    float* sr = zs + (size_t)i * R;
+    const int t = t0 + i;
+    float mx = -INFINITY;
+    for (int e = 0; e < R; ++e) mx = fmaxf(mx, sr[e]);
+    float sum = 0.f;
+    for (int e = 0; e < R; ++e) {
+        const float v = expf(sr[e] - mx);
+        sr[e] = v;
+        sum += v;
+    }
+    const float inv = 1.0f / sum;
+    for (int e = 0; e < R; ++e) sr[e] *= inv;
+    const int gs = R / groups;
+    unsigned long long open = ~0ull;
+    if (keep < groups) {
+        open = 0ull;
+        for (int r = 0; r < keep; ++r) {
+            int best = -1;
+            float best_v = -INFINITY;
+            for (int g = 0; g < groups; ++g) {
+                if ((open >> g) & 1ull) continue;
+                float gv = -INFINITY;
+                for (int e = g * gs; e < (g + 1) * gs; ++e) gv = fmaxf(gv, sr[e] + (correction ? correction[e] : 0.f));
+                if (best < 0 || gv > best_v) {
+                    best = g;
+                    best_v = gv;
+                }
+            }
+            open |= 1ull << best;
+        }
+    }
+    for (int r = 0; r < top; ++r) {
+        int best = -1;
+        float best_v = -INFINITY;
+        for (int e = 0; e < R; ++e) {
+            const float se = sr[e];
+            if (se < 0.f || !((open >> (e / gs)) & 1ull)) continue;
+            const float c = se + (correction ? correction[e] : 0.f);
+            if (best < 0 || c > best_v) {
+                best = e;
+                best_v = c;
+            }
+        }
+        choice[(size_t)t * top + r] = best;
+        weight[(size_t)t * top + r] = sr[best] * scale;
+        sr[best] = -1.0f - sr[best];
+    }
+}
+
+extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float* router, const float* correction, int N, int K,
+                                int R, int groups, int keep, int top, float scale, int* choice, float* weight,
+                                hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && K > 0 && R > 0 && R <= ROUTE_MAX, "route_rows: %d router outputs (1 to %d)", R, ROUTE_MAX);
+    AGAVE_CHECK(groups > 0 && groups <= 64 && R % groups == 0, "route_rows: %d outputs in %d groups (equal groups, at most 64)", R, groups);
+    AGAVE_CHECK(keep > 0 && keep <= groups, "route_rows: %d of %d groups kept", keep, groups);
+    AGAVE_CHECK(top > 0 && top <= keep * (R / groups), "route_rows: %d chosen of %d that are open", top, keep * (R / groups));
+    AGAVE_CHECK(x && router && choice && weight && ldx >= K, "route_rows: bad buffers");
+    if (N == 0) return 0;
+    const int blocks = (N + ROUTE_ROWS - 1) / ROUTE_ROWS;
+    const size_t lds = (size_t)ROUTE_ROWS * R * sizeof(float);
+    const int threads = blocks < 128 ? 1024 : 256;
+    const bool wide = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 32) == 0 && ((uintptr_t)router % 32) == 0;
+    if (dtype == AGAVE_F32) {
+        if (wide)
+            route_rows_kernel<float, true><<<blocks, threads, lds, stream>>>((const float*)x, ldx, router, correction, N, K, R, groups,
+                                                                             keep, top, scale, choice, weight);
+        else
+            route_rows_kernel<float, false><<<blocks, threads, lds, stream>>>((const float*)x, ldx, router, correction, N, K, R, groups,
+                                                                              keep, top, scale, choice, weight);
+    } else if (dtype == AGAVE_BF16) {
+        if (wide)
+            route_rows_kernel<bf16, true><<<blocks, threads, lds, stream>>>((const bf16*)x, ldx, router, correction, N, K, R, groups,
+                                                                            keep, top, scale, choice, weight);
+        else
+            route_rows_kernel<bf16, false><<<blocks, threads, lds, stream>>>((const bf16*)x, ldx, router, correction, N, K, R, groups,
+                                                                             keep, top, scale, choice, weight);
+    } else
+        AGAVE_CHECK(false, "route_rows: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("route_rows");
+    return 0;
+}
+
 // ------------------------------------------------------------------ activations of the experts' gates
 __device__ __forceinline__ float expert_act(float x, int act) {
     switch (act) {
@@ -219,5 +371,185 @@ extern "C" int agave_routed_combine(int dtype, const float* y, const int* place,
     else
         AGAVE_CHECK(false, "routed_combine: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("routed_combine");
+    return 0;
+}
+
+// ------------------------------------------------------------------ the pairs sorted by expert
+// One workgroup.  Every expert's pairs get a run of whole tiles of TM sorted rows (the last one padded):
+//   place[p]        sorted row of pair p (-1: the pair's choice is an identity expert)
+//   sorted_pair[r]  pair in sorted row r (-1: padding)
+//   tile_expert[t]  expert of tile t (-1: no such tile)
+// The order of an expert's pairs among themselves is whatever the atomics make it; every row's result is
+// its own, so nothing depends on it.
+__global__ __launch_bounds__(1024) void route_sort_kernel(const int* __restrict__ choice, int P, int E, int TM, int cap,
+                                                          int max_tiles, int* __restrict__ place,
+                                                          int* __restrict__ sorted_pair, int* __restrict__ tile_expert) {
+    __shared__ int counts[ROUTE_MAX];
+    __shared__ int first_row[ROUTE_MAX];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) counts[e] = 0;
+    for (int r = tid; r < cap; r += blockDim.x) sorted_pair[r] = -1;
+    for (int t = tid; t < max_tiles; t += blockDim.x) tile_expert[t] = -1;
+    __syncthreads();
+    for (int p = tid; p < P; p += blockDim.x) {
+        const int e = choice[p];
+        place[p] = (e >= 0 && e < E) ? atomicAdd(&counts[e], 1) : -1;        // for now: the pair's rank within its expert
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int tile = 0;
+        for (int e = 0; e < E; ++e) {
+            first_row[e] = tile * TM;
+            const int n = (counts[e] + TM - 1) / TM;
+            for (int i = 0; i < n && tile + i < max_tiles; ++i) tile_expert[tile + i] = e;
+            tile += n;
+        }
+    }
+    __syncthreads();
+    for (int p = tid; p < P; p += blockDim.x) {
+        const int e = choice[p];
+        if (e >= 0 && e < E) {
+            const int r = first_row[e] + place[p];
+            if (r < cap) {
+                place[p] = r;
+                sorted_pair[r] = p;
+            } else {
+                place[p] = -1;          // (cannot happen: cap holds every pair and every expert's padding)
+            }
+        }
+    }
+}
+
+extern "C" int agave_route_sort(const int* choice, int P, int E, int TM, int cap, int max_tiles, int* place, int* sorted_pair,
+                                int* tile_expert, hipStream_t stream) {
+    AGAVE_CHECK(P >= 0 && E > 0 && E <= ROUTE_MAX && (TM == 16 || TM == 64), "route_sort: bad sizes P=%d E=%d TM=%d", P, E, TM);
+    AGAVE_CHECK(max_tiles >= (P + TM - 1) / TM + E && cap >= max_tiles * TM, "route_sort: %d tiles of %d rows do not hold %d pairs of %d experts",
+                max_tiles, TM, P, E);
+    AGAVE_CHECK(choice && place && sorted_pair && tile_expert, "route_sort: null buffer");
+    if (P == 0) return 0;
+    route_sort_kernel<<<1, 1024, 0, stream>>>(choice, P, E, TM, cap, max_tiles, place, sorted_pair, tile_expert);
+    AGAVE_LAUNCH_CHECK("route_sort");
+    return 0;
+}
+
+// ------------------------------------------------------------------ the experts' products on the matrix cores
+// A workgroup takes one tile of TM = 16 MI sorted rows (one expert) and 64 NJ output columns, 16 NJ a wave; both operands
+// come straight from memory in the order v_mfma_f32_16x16x32_bf16 reads them (a lane's eight neighbours along K are
+// 16 bytes of a row of X or of W[e]).  GATED: two products (gate and up) side by side, ending in act(gate) * up,
+// rows gathered from X through the sorted pairs; otherwise one product of the sorted inner rows, 32-bit out.
+template <int MI, int NJ, bool GATED>
+__global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __restrict__ x, long ldx, const int* __restrict__ sorted_pair,
+                                                                  const int* __restrict__ tile_expert, const bf16* __restrict__ w0,
+                                                                  const bf16* __restrict__ w1, void* __restrict__ out_, int top,
+                                                                  int n_out, int K, int act) {
+    const int e = tile_expert[blockIdx.x];
+    if (e < 0) return;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int c = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * 16 * MI;
+    const int col0 = blockIdx.y * (64 * NJ) + w * (16 * NJ);
+    if (col0 >= n_out) return;
+    // A rows: 16 i + c of the tile
+    const bf16* arow[MI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        const int r = row0 + 16 * i + c;
+        if (GATED) {
+            const int p = sorted_pair[r];
+            arow[i] = x + (size_t)(p >= 0 ? p / top : 0) * ldx + 8 * g;       // (a padding row computes on row 0 and is never read)
+        } else {
+            arow[i] = x + (size_t)r * ldx + 8 * g;
+        }
+    }
+    // B rows: output columns col0 + 16 j + c of expert e (clamped; columns past the end are not stored)
+    const bf16* b0[NJ];
+    const bf16* b1[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        int col = col0 + 16 * j + c;
+        if (col >= n_out) col = n_out - 1;
+        b0[j] = w0 + ((size_t)e * n_out + col) * K + 8 * g;
+        b1[j] = GATED ? w1 + ((size_t)e * n_out + col) * K + 8 * g : nullptr;
+    }
+    f32x4_t acc0[MI][NJ], acc1[MI][GATED ? NJ : 1];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            acc0[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            if (GATED) acc1[i][GATED ? j : 0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        // (loads without conditions, from inside the row; a lane past the row's end reads its start and is emptied)
+        const bool in = k0 + 8 * g < K;
+        const int at = in ? k0 : -8 * g;
+        frag16 a[MI], bw0[NJ], bw1[NJ];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) a[i].u = *reinterpret_cast<const uint4*>(arow[i] + at);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            bw0[j].u = *reinterpret_cast<const uint4*>(b0[j] + at);
+            if (GATED) bw1[j].u = *reinterpret_cast<const uint4*>(b1[j] + at);
+        }
+        if (!in) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i) a[i].u = make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                acc0[i][j] = mfma_16x16x32(a[i], bw0[j], acc0[i][j]);
+                if (GATED) acc1[i][GATED ? j : 0] = mfma_16x16x32(a[i], bw1[j], acc1[i][GATED ? j : 0]);
+            }
+    }
+    // D[i][j]: lane holds rows 4 g + e4 of the row block, column c of the column block
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int col = col0 + 16 * j + c;
+            if (col >= n_out) continue;
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const size_t r = (size_t)row0 + 16 * i + 4 * g + e4;
+                if (GATED) {
+                    // (gate and up are rounded to the rows' type before the activation, as the plain kernel does)
+                    const float gt = bf16_to_f32(f32_to_bf16(acc0[i][j][e4])), up = bf16_to_f32(f32_to_bf16(acc1[i][GATED ? j : 0][e4]));
+                    ((bf16*)out_)[r * n_out + col] = f32_to_bf16(expert_act(gt, act) * up);
+                } else {
+                    ((float*)out_)[r * n_out + col] = acc0[i][j][e4];
+                }
+            }
+        }
+}
+
+// act_rows [cap, ff] bfloat16 and y [cap, hidden] float32 hold sorted rows (see route_sort)
+extern "C" int agave_routed_experts_mfma(const void* x, long ldx, const int* sorted_pair, const int* tile_expert, const void* wg,
+                                         const void* wu, const void* wd, void* act_rows, float* y, int TM, int max_tiles, int top,
+                                         int E, int ff, int hidden, int act, hipStream_t stream) {
+    AGAVE_CHECK(max_tiles > 0 && top > 0 && E > 0 && ff > 0 && hidden > 0 && (TM == 16 || TM == 64), "routed_experts_mfma: bad sizes");
+    AGAVE_CHECK(act >= 0 && act < 4, "routed_experts_mfma: unknown activation %d", act);
+    AGAVE_CHECK(hidden % 8 == 0 && ff % 8 == 0 && ldx % 8 == 0, "routed_experts_mfma: sizes must be multiples of 8 (hidden %d, ff %d)", hidden, ff);
+    AGAVE_CHECK(x && sorted_pair && tile_expert && wg && wu && wd && act_rows && y, "routed_experts_mfma: null buffer");
+    AGAVE_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wg % 16) == 0 && ((uintptr_t)wu % 16) == 0 && ((uintptr_t)wd % 16) == 0 &&
+                ((uintptr_t)act_rows % 16) == 0, "routed_experts_mfma: buffers must be aligned to 16 bytes");
+    // tiles of 64 rows take 64 columns a wave (an operand that was loaded serves more multiplications), tiles of
+    // 16 rows, which stream their weights once, 32
+    const int cols = TM == 64 ? 256 : 128;
+    const dim3 g1(max_tiles, (ff + cols - 1) / cols), g2(max_tiles, (hidden + cols - 1) / cols);
+    AGAVE_CHECK(g1.y <= 65535 && g2.y <= 65535, "routed_experts_mfma: too many columns for the grid");
+    if (TM == 64) {
+        routed_product_mfma_kernel<4, 4, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
+                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act);
+        routed_product_mfma_kernel<4, 4, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
+                                                                     nullptr, y, top, hidden, ff, act);
+    } else {
+        routed_product_mfma_kernel<1, 2, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
+                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act);
+        routed_product_mfma_kernel<1, 2, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
+                                                                     nullptr, y, top, hidden, ff, act);
+    }
+    AGAVE_LAUNCH_CHECK("routed_experts_mfma");
     return 0;
 }

@@ -14,6 +14,9 @@ MAX_OUTPUTS = 1024
 kernels.register_signatures(LIBRARY, {
     "agave_route_topk": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
     "agave_routed_experts_plain": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "agave_route_rows": [_I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+    "agave_route_sort": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
+    "agave_routed_experts_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "agave_routed_combine": [_I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 
@@ -83,3 +86,75 @@ def combine(y: Optional[torch.Tensor], place: Optional[torch.Tensor], choice: to
     _i32(place, "place", n * top)
     library.call(_lib(), "agave_routed_combine", dt(x), ptr(y), ptr(place), ptr(choice), ptr(weight), ptr(x), ldx, ptr(shared),
                  lds, ptr(out), ldo, n, top, n_experts, hidden, stream())
+
+
+def tile_plan(n_pairs: int, n_experts: int):
+    """(rows a tile, tiles at most, sorted rows at most) of the sorted list of ``n_pairs`` pairs: tiles of 64 rows
+    where an expert gets some 32 pairs or more on average, of 16 otherwise; every expert's run of rows is padded to
+    whole tiles, so there are at most ``ceil(pairs / rows) + experts`` tiles."""
+    tm = 64 if n_pairs >= 32 * n_experts else 16
+    tiles = (n_pairs + tm - 1) // tm + n_experts
+    return tm, tiles, tiles * tm
+
+
+def mfma_ok(x: torch.Tensor, ff: int) -> bool:
+    """Whether the matrix-core kernels take these rows (bfloat16, sizes that are multiples of 8, aligned)."""
+    return (x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and ff % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0)
+
+
+def route_sort(choice: torch.Tensor, n_experts: int, tm: int, tiles: int, place: torch.Tensor, sorted_pair: torch.Tensor,
+               tile_expert: torch.Tensor) -> None:
+    """Sort the pairs by expert on the device: ``place[p]`` the sorted row of pair p (-1 for an identity expert),
+    ``sorted_pair[r]`` the pair in sorted row r (-1: padding), ``tile_expert[t]`` the expert of tile t (-1: none)."""
+    _dev(choice, place, sorted_pair, tile_expert)
+    p = choice.numel()
+    _i32(choice, "choice")
+    _i32(place, "place", p)
+    _i32(sorted_pair, "sorted_pair", tiles * tm)
+    _i32(tile_expert, "tile_expert", tiles)
+    library.call(_lib(), "agave_route_sort", ptr(choice), p, n_experts, tm, tiles * tm, tiles, ptr(place), ptr(sorted_pair),
+                 ptr(tile_expert), stream())
+
+
+def experts_mfma(x: torch.Tensor, sorted_pair: torch.Tensor, tile_expert: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
+                 w_down: torch.Tensor, act_rows: torch.Tensor, y: torch.Tensor, tm: int, tiles: int, top: int, activation: int) -> None:
+    """The experts' products over the sorted rows on the matrix cores: ``act_rows`` [tiles * tm, ff] bfloat16 and
+    ``y`` [tiles * tm, hidden] float32 receive sorted rows (padding rows hold nothing of use)."""
+    _dev(x, sorted_pair, tile_expert, w_gate, w_up, w_down, act_rows, y)
+    n, hidden = x.shape
+    e, ff, k = w_gate.shape
+    if k != hidden or w_up.shape != w_gate.shape or w_down.shape != (e, hidden, ff):
+        raise ValueError("experts: weights must be [E, ff, hidden], [E, ff, hidden] and [E, hidden, ff]")
+    for w in (w_gate, w_up, w_down):
+        if w.dtype != torch.bfloat16 or not w.is_contiguous():
+            raise TypeError("experts: the matrix-core kernels take contiguous bfloat16 weights")
+    if not mfma_ok(x, ff):
+        raise ValueError("experts: rows that the matrix-core kernels do not take")
+    cap = tiles * tm
+    if act_rows.dtype != torch.bfloat16 or not act_rows.is_contiguous() or act_rows.shape != (cap, ff):
+        raise ValueError(f"experts: inner rows must be bfloat16 [{cap}, {ff}]")
+    if y.dtype != torch.float32 or not y.is_contiguous() or y.shape != (cap, hidden):
+        raise ValueError(f"experts: y must be float32 [{cap}, {hidden}]")
+    _i32(sorted_pair, "sorted_pair", cap)
+    _i32(tile_expert, "tile_expert", tiles)
+    library.call(_lib(), "agave_routed_experts_mfma", ptr(x), x.stride(0), ptr(sorted_pair), ptr(tile_expert), ptr(w_gate),
+                 ptr(w_up), ptr(w_down), ptr(act_rows), ptr(y), tm, tiles, top, e, ff, hidden, activation, stream())
+
+
+def route_rows(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
+               scale: float, choice: torch.Tensor, weight: torch.Tensor) -> None:
+    """The router's 32-bit product ``x router^T`` and :func:`route_topk`'s choice in one kernel (the logits never
+    leave the compute unit).  ``router`` is float32 [R, width]; ``x`` [N, width] in either element type."""
+    _dev(x, router, correction, choice, weight)
+    n, k = x.shape
+    ldx = _rows(x, "x")
+    if router.dtype != torch.float32 or router.dim() != 2 or router.shape[1] != k or not router.is_contiguous():
+        raise ValueError(f"route_rows: the router must be contiguous float32 [outputs, {k}]")
+    r = router.shape[0]
+    _f32vec(correction, "correction", r)
+    _i32(choice, "choice", n * top)
+    if weight.dtype != torch.float32 or not weight.is_contiguous() or weight.numel() < n * top:
+        raise ValueError("route_rows: weight must be contiguous float32 [N, top]")
+    library.call(_lib(), "agave_route_rows", dt(x), ptr(x), ldx, ptr(router), ptr(correction), n, k, r, groups, keep, top,
+                 float(scale), ptr(choice), ptr(weight), stream())

@@ -76,20 +76,29 @@ class RoutedFfn:
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         s, ws = self.spec, self.env.workspace
         n, r, top = x.shape[0], self.n_outputs, s.top
-        logits = ws.get("router_logits", n, r, torch.float32)
-        kernels.gemm_plain(x, self.router, logits)
-        scratch = ws.get("router_scores", n, r, torch.float32)
         choice = ws.get("router_choice", n, top, torch.int32)
         weight = ws.get("router_weight", n, top, torch.float32)
-        routed.route_topk(logits, self.correction, scratch, s.groups, s.keep_groups, top, s.route_scale, choice, weight)
-        y = None
-        if s.n_experts:
+        # the router's 32-bit product and the choice in one kernel
+        routed.route_rows(x, self.router, self.correction, s.groups, s.keep_groups, top, s.route_scale, choice, weight)
+        y = place = None
+        if s.n_experts and self.w_gate.dtype == torch.bfloat16 and routed.mfma_ok(x, s.intermediate):
+            # the pairs sorted by expert on the device, then the experts' products tile by tile on the matrix cores
+            tm, tiles, cap = routed.tile_plan(n * top, s.n_experts)
+            place = ws.get("expert_place", n * top, 1, torch.int32).view(-1)
+            sorted_pair = ws.get(f"expert_sorted{tm}", cap, 1, torch.int32).view(-1)
+            tile_expert = ws.get(f"expert_tiles{tm}", tiles, 1, torch.int32).view(-1)
+            routed.route_sort(choice.view(-1), s.n_experts, tm, tiles, place, sorted_pair, tile_expert)
+            act_rows = ws.get("expert_act", cap, s.intermediate, x.dtype)
+            y = ws.get("expert_rows", cap, s.hidden, torch.float32)
+            routed.experts_mfma(x, sorted_pair, tile_expert, self.w_gate, self.w_up, self.w_down, act_rows, y, tm, tiles, top,
+                                self.act)
+        elif s.n_experts:
             act_rows = ws.get("expert_act", n * top, s.intermediate, x.dtype)
             y = ws.get("expert_rows", n * top, s.hidden, torch.float32)
             routed.experts_plain(x, choice.view(-1), self.w_gate, self.w_up, self.w_down, act_rows, y, top, self.act)
         shared = self.shared.forward(x, step, slices_ok=False, tag="shared_ffn") if self.shared is not None else None
         out = ws.get("routed_out", n, s.hidden, x.dtype)
-        routed.combine(y, None, choice.view(-1), weight.view(-1), x, shared, out, top, s.n_experts)
+        routed.combine(y, place, choice.view(-1), weight.view(-1), x, shared, out, top, s.n_experts)
         return out
 
 

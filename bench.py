@@ -23,9 +23,9 @@ The other published shapes:
 
 Another design beside the closest Gemma 3 shape of equal size (not the default run):
 
-    python bench.py --design rilenex [--design-size small|medium|large] [--design-layers 8]
+    python bench.py --design rilenex|gusedra [--design-size small|medium|large] [--design-layers 8]
 
-prints one JSON line with, for the Rilenex decoder and for a Gemma 3 decoder of the same width, depth,
+prints one JSON line with, for that decoder and for a Gemma 3 decoder of the same width, depth,
 heads and about as many weights: tokens a second of a 2,048-token prompt and of decode steps at
 batch 8 and 1, and the time of every kind of kernel in one prompt and in one decode step.
 """
@@ -218,6 +218,31 @@ def rilenex_config(size: str, layers: int) -> dict:
             "layers": [par if i % 4 == 2 else hgrn2 for i in range(layers)]}
 
 
+def gusedra_config(size: str, layers: int) -> dict:
+    """Layers of both attention mixers in turn (a learned bias over buckets with kept first positions and a gate;
+    slopes with sinks), every fourth one reading the keys and values of the layer before it; feed-forwards in
+    turn dense (the square of ReLU) and routed (16 experts of a quarter of the dense inner size plus two identity
+    experts in 2 groups of 9, 4 of them a token, and a shared expert): a token's routed layer computes as much as
+    a dense one.  Heads of 128, windows of 1,024 as the Gemma 3 shape beside it."""
+    e, ff, h, g, d, _, _ = DESIGN_SIZES[size]
+    def mixer(kind, i):
+        m = {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}}
+        if kind == "attention_2":
+            m["mask"]["keep_first"] = 4
+            m["bias_max"] = 2048
+        elif i % 4 == 3:
+            m["kv_from"] = i - 2
+        return m
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4},
+           "router": {"experts": 16, "identity": 2, "top": 4, "scale": 2.0, "groups": {"count": 2, "keep": 1}}}
+    out = []
+    for i in range(layers):
+        kind = "attention_2" if i % 2 == 0 else "attention"
+        out.append({"type": kind, "mixer": mixer(kind, i), "mlp": moe if i % 2 else dense})
+    return {"architecture": "Gusedra", "vocab": 32768, "width": e, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": out}
+
+
 def gemma_like_config(size: str, layers: int) -> dict:
     """The same width, depth and heads as a Gemma 3 decoder; its gated feed-forward has three matrices,
     so two thirds of the inner size give as many weights."""
@@ -266,7 +291,8 @@ def compare_designs(args) -> int:
     result = {"metric": f"{args.design} beside Gemma 3 at equal size ({size}, {layers} layers): tokens/s", "unit": "tokens/s",
               "dtype": "bf16", "data": "synthetic: uniform-random token ids, random weights", "sizes": DESIGN_SIZES[size],
               "peaks_measured": measured_peaks()}
-    for name, cfg in ((args.design, rilenex_config(size, layers)), ("gemma3_equal_size", gemma_like_config(size, layers))):
+    design = {"rilenex": rilenex_config, "gusedra": gusedra_config}[args.design](size, layers)
+    for name, cfg in ((args.design, design), ("gemma3_equal_size", gemma_like_config(size, layers))):
         engine = Engine.from_random(cfg, seed=0, dtype="bfloat16", max_slots=batch, max_context=context,
                                     cache_tokens=batch * (PREFILL_LEN + 512), device="cuda:0")
         rec = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3)}
@@ -305,7 +331,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
-    ap.add_argument("--design", choices=["rilenex"], help="measure this design beside a Gemma 3 decoder of equal size")
+    ap.add_argument("--design", choices=["rilenex", "gusedra"], help="measure this design beside a Gemma 3 decoder of equal size")
     ap.add_argument("--design-size", default="medium", choices=sorted(DESIGN_SIZES))
     ap.add_argument("--design-layers", type=int, default=8)
     args = ap.parse_args()
