@@ -79,8 +79,14 @@ class KVCache:
             if k.layout == "tiles" and k.v_head_dim not in (None, k.head_dim):
                 raise CacheError("pages in tile order hold keys and values of one size; a mixer with narrower "
                                  "values asks for the layout 'rows'")
-        self.packed: List[bool] = [k.layout == "tiles" and dtype == torch.bfloat16 and k.head_dim % 16 == 0
-                                   and k.head_dim <= 256 for k in self.group_keys]
+        # ("rows_vt" in bfloat16 with a key size that is a multiple of 8 and a value size that is a multiple of 16:
+        # the same, in the order the biased attention's matrix-core kernel reads its operands)
+        self.packed: List[bool] = [
+            dtype == torch.bfloat16 and k.head_dim <= 256 and
+            ((k.layout == "tiles" and k.head_dim % 16 == 0) or
+             (k.layout == "rows_vt" and k.head_dim % 8 == 0 and (k.v_head_dim or k.head_dim) % 16 == 0
+              and (k.v_head_dim or k.head_dim) <= 256))
+            for k in self.group_keys]
         for key, mems, packed in zip(self.group_keys, members, self.packed):
             n = pages_per_group[key]
             hd_k = (key.head_dim + 31) // 32 * 32 if packed else key.head_dim
@@ -93,7 +99,7 @@ class KVCache:
                 self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, vd), dtype=dtype, device=device))
             elif key.layout == "rows_vt":
                 vd = key.v_head_dim or key.head_dim
-                self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, key.head_dim), dtype=dtype, device=device))
+                self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, hd_k), dtype=dtype, device=device))
                 self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, vd, PAGE), dtype=dtype, device=device))
             else:
                 self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, hd_k), dtype=dtype, device=device))

@@ -10,7 +10,8 @@
 //   * a gate on the output rows: out *= sigmoid(gate), element by element.
 // Scores, bias, softmax and the sums over values are 32-bit in every element type.
 //
-// Cache pages: K [page][kv head][64 rows][hd]; V transposed [page][kv head][vd][64 rows].
+// Cache pages: K [page][kv head][64 rows][hd]; V transposed [page][kv head][vd][64 rows]; or both in the order the
+// matrix-core kernel reads its operands (below), which is how a bfloat16 cache holds them where the sizes allow.
 // Position j of sequence b lies in row j % 64 of the page in column col(j / 64) of table[b]:
 //   col(i) = i < head ? i : head + i - base[b]        (base[b] >= head)
 // so the first `head` columns are the pages that hold the kept first positions, and the
@@ -24,13 +25,28 @@
 
 __device__ __forceinline__ int page_col(int pi, int pbase, int head) { return pi < head ? pi : head + pi - pbase; }
 
+// Pages in operand order (bfloat16, for the matrix-core kernel): a (page, kv head) block of keys is
+// [4 key blocks][ksl = ceil(hd / 32) steps][64 lanes][8], lane c + 16 g of (kb, ks) holding elements
+// 32 ks + 8 g .. + 8 of key key_of(kb, c) (see the kernel); a block of values is [vd / 16][2][64][8], lane
+// c + 16 g of (nb, h) holding keys 32 h + 8 g .. + 8 of value column 16 nb + c.  A wave reads an operand
+// of either with one load of a kilobyte in a row.  Where the head size is no multiple of 32 the last
+// step's upper lanes stay zero (pages start out zeroed and nothing is ever written there).
+__device__ __forceinline__ size_t k_operand_at(int r, int d, int ksl) {
+    const int h = r >> 5, g4 = (r & 31) >> 3, sub = r & 7;
+    const int kb = 2 * h + (sub >> 2), i = 4 * g4 + (sub & 3);
+    return ((size_t)(kb * ksl + (d >> 5)) * 64 + i + 16 * ((d & 31) >> 3)) * 8 + (d & 7);
+}
+__device__ __forceinline__ size_t v_operand_at(int d, int r) {
+    return ((size_t)((d >> 4) * 2 + (r >> 5)) * 64 + (d & 15) + 16 * ((r & 31) >> 3)) * 8 + (r & 7);
+}
+
 // ------------------------------------------------------------------ k and v rows into their pages
 template <typename T>
 __global__ void kv_append_rows_kernel(const T* __restrict__ k, long ldk, const T* __restrict__ v, long ldv,
                                       T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ table,
                                       int width, const int* __restrict__ base, int head, int n_pages,
                                       const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int nkv, int hd,
-                                      int vd) {
+                                      int vd, int packed) {
     const int t = blockIdx.x;
     const int b = tok_seq[t], p = tok_pos[t];
     const int col = page_col(p / AGAVE_PAGE, base[b], head);
@@ -38,34 +54,38 @@ __global__ void kv_append_rows_kernel(const T* __restrict__ k, long ldk, const T
     const long pg = table[(size_t)b * width + col];
     if (pg < 0 || pg >= n_pages) return;
     const int row = p % AGAVE_PAGE;
+    const int ksl = (hd + 31) / 32;
+    const size_t kblock = packed ? (size_t)AGAVE_PAGE * ksl * 32 : (size_t)AGAVE_PAGE * hd;
     for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
         const int g = i / hd, d = i % hd;
-        k_pages[(((size_t)pg * nkv + g) * AGAVE_PAGE + row) * hd + d] = k[(size_t)t * ldk + i];
+        k_pages[((size_t)pg * nkv + g) * kblock + (packed ? k_operand_at(row, d, ksl) : (size_t)row * hd + d)] = k[(size_t)t * ldk + i];
     }
     for (int i = threadIdx.x; i < nkv * vd; i += blockDim.x) {
         const int g = i / vd, d = i % vd;
-        v_pages[(((size_t)pg * nkv + g) * vd + d) * AGAVE_PAGE + row] = v[(size_t)t * ldv + i];
+        v_pages[((size_t)pg * nkv + g) * vd * AGAVE_PAGE + (packed ? v_operand_at(d, row) : (size_t)d * AGAVE_PAGE + row)] =
+            v[(size_t)t * ldv + i];
     }
 }
 
 extern "C" int agave_kv_append_rows(int dtype, const void* k, long ldk, const void* v, long ldv, void* k_pages,
                                     void* v_pages, const int* table, int width, const int* base, int head, int n_pages,
-                                    const int* tok_seq, const int* tok_pos, int N, int nkv, int hd, int vd,
+                                    const int* tok_seq, const int* tok_pos, int N, int nkv, int hd, int vd, int packed,
                                     hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && nkv > 0 && hd > 0 && vd > 0, "kv_append_rows: bad sizes N=%d nkv=%d hd=%d vd=%d", N, nkv, hd, vd);
     AGAVE_CHECK(k && v && k_pages && v_pages && table && base && tok_seq && tok_pos && width > 0 && n_pages > 0,
                 "kv_append_rows: null buffer or empty table");
     AGAVE_CHECK(ldk >= (long)nkv * hd && ldv >= (long)nkv * vd, "kv_append_rows: a row stride is too small");
     AGAVE_CHECK(head >= 0, "kv_append_rows: negative count of kept pages");
+    AGAVE_CHECK(!packed || (dtype == AGAVE_BF16 && hd % 8 == 0 && vd % 16 == 0), "kv_append_rows: pages in operand order hold bfloat16, keys in steps of 8 and values in steps of 16");
     if (N == 0) return 0;
     if (dtype == AGAVE_F32)
         kv_append_rows_kernel<float><<<N, 128, 0, stream>>>((const float*)k, ldk, (const float*)v, ldv, (float*)k_pages,
                                                             (float*)v_pages, table, width, base, head, n_pages, tok_seq,
-                                                            tok_pos, nkv, hd, vd);
+                                                            tok_pos, nkv, hd, vd, 0);
     else if (dtype == AGAVE_BF16)
         kv_append_rows_kernel<bf16><<<N, 128, 0, stream>>>((const bf16*)k, ldk, (const bf16*)v, ldv, (bf16*)k_pages,
                                                            (bf16*)v_pages, table, width, base, head, n_pages, tok_seq,
-                                                           tok_pos, nkv, hd, vd);
+                                                           tok_pos, nkv, hd, vd, packed);
     else
         AGAVE_CHECK(false, "kv_append_rows: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("kv_append_rows");
@@ -87,6 +107,7 @@ struct BiasedArgs {
     int bias_mode;                       // 0 none, 1 slopes, 2 table over distances
     const float* bias; int bias_len;     // slopes [nh], or table [nh][bias_len]
     const float* sink;                   // [nh] or null
+    int packed;                          // the pages are in operand order
 };
 
 __device__ __forceinline__ float score_bias(const BiasedArgs& A, int h, int dist) {
@@ -150,9 +171,15 @@ __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
             const bool valid = j >= j_lo && j <= j_hi && pg >= 0;
             float s = -INFINITY;
             if (valid) {
-                const T* kr = k_pages + (((size_t)pg * nkv + kvh) * AGAVE_PAGE + (j % AGAVE_PAGE)) * hd;
                 float dot = 0.f;
-                for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], ld(kr + d), dot);
+                if (A.packed) {
+                    const int ksl = (hd + 31) / 32;
+                    const T* kblk = k_pages + ((size_t)pg * nkv + kvh) * AGAVE_PAGE * ksl * 32;
+                    for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], ld(kblk + k_operand_at(j % AGAVE_PAGE, d, ksl)), dot);
+                } else {
+                    const T* kr = k_pages + (((size_t)pg * nkv + kvh) * AGAVE_PAGE + (j % AGAVE_PAGE)) * hd;
+                    for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], ld(kr + d), dot);
+                }
                 s = dot * A.scale + score_bias(A, h, p - j);
             }
             const float cmax = block_max(s, red);
@@ -171,10 +198,11 @@ __global__ __launch_bounds__(256) void attn_biased_plain_kernel(BiasedArgs A) {
                     for (int pi = 0; pi < BCHUNK / AGAVE_PAGE; ++pi) {
                         const long vp = page_of[pi];
                         if (vp < 0) continue;
-                        const T* vr = v_pages + (((size_t)vp * nkv + kvh) * vd + d) * AGAVE_PAGE;
+                        const T* vblk = v_pages + ((size_t)vp * nkv + kvh) * vd * AGAVE_PAGE;
+                        const T* vr = vblk + (size_t)d * AGAVE_PAGE;
                         for (int r = 0; r < AGAVE_PAGE; ++r) {
                             const float w = sc[pi * AGAVE_PAGE + r];
-                            if (w != 0.f) sum = fmaf(w, ld(vr + r), sum);   // rows out of range hold w == 0
+                            if (w != 0.f) sum = fmaf(w, ld(A.packed ? vblk + v_operand_at(d, r) : vr + r), sum);   // rows out of range hold w == 0
                         }
                     }
                     acc[a] = acc[a] * alpha + sum;
@@ -218,10 +246,11 @@ extern "C" int agave_attn_biased_plain(int dtype, const void* q, long ldq, void*
                                        const void* k_pages, const void* v_pages, const int* table, int width,
                                        const int* base, int head, int n_pages, const int* tok_seq, const int* tok_pos, int N,
                                        int nh, int nkv, int hd, int vd, float scale, int window, int keep_first,
-                                       int bias_mode, const float* bias, int bias_len, const float* sink,
+                                       int bias_mode, const float* bias, int bias_len, const float* sink, int packed,
                                        hipStream_t stream) {
     BiasedArgs A{q, ldq, out, ldo, gate, ldg, k_pages, v_pages, table, width, base, head, n_pages, tok_seq, tok_pos,
-                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink};
+                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, packed};
+    AGAVE_CHECK(!packed || dtype == AGAVE_BF16, "attn_biased: pages in operand order hold bfloat16");
     if (check_biased(A, N)) return -1;
     if (N == 0) return 0;
     if (dtype == AGAVE_F32)
@@ -241,10 +270,13 @@ extern "C" int agave_attn_biased_plain(int dtype, const void* q, long ldq, void*
 // v_mfma_f32_16x16x32_bf16, so that a lane holds scores of one column a block only: the column's running
 // maximum, sum and rescaling factor are the lane's own (and its three partners' in the other lane
 // groups), and the probabilities go from the score registers straight into the B operand of
-// O^T += V^T P^T, whose keys are taken in the order the score registers hold them (the A operand,
-// a value column's keys from the transposed page, is read in that order: two 8-byte loads).  A key or
-// value operand that was loaded serves all NC column blocks.
-//   S^T tile of key block kb: lane l holds keys 16 kb + 4 (l / 16) + e, e = 0..3, of column l % 16
+// O^T += V^T P^T.  A key or value operand that was loaded serves all NC column blocks.
+// Which key a row of a score tile stands for is the kernel's choice; row i of key block kb is key
+//   key_of(kb, i) = 32 (kb / 2) + 8 (i / 4) + 4 (kb % 2) + i % 4
+// of the page, so that a lane group's scores of two neighbouring key blocks are eight neighbouring keys, the
+// eight that a lane's B operand of one step of O^T += V^T P^T holds, and the matching A operand is 16 bytes
+// of a value column's row in the transposed page:
+//   S^T tile of key block kb: lane l holds keys 32 (kb / 2) + 8 (l / 16) + 4 (kb % 2) + e, e = 0..3, of column l % 16
 //   O^T block nb:             lane l holds value columns 16 nb + 4 (l / 16) + e of column l % 16
 // Many rows: a workgroup is four waves with 16 NC rows each, all pages each.  One row: the workgroup's
 // waves (four or eight) share the pages of one (row, key head) and wave 0 merges their partial results
@@ -309,6 +341,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         pmax = A.tok_pos[min(wr0 + WROWS, r1) - 1];
     }
     const int kvh = head / per;
+    const int ksl = (hd + 31) / 32;                 // steps along the head that the pages hold
     const int W = A.window, keep = A.keep_first;
     const int lo = W > 0 ? max(0, pmin - W + 1) : 0;
     const int first_win = lo / AGAVE_PAGE;
@@ -366,7 +399,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         pg = pg_next;
         if (pg_now < 0) continue;
         const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
-        const bf16* kb_ = (const bf16*)A.k_pages + ((size_t)pg_now * nkv + kvh) * AGAVE_PAGE * hd;
+        const bf16* kb_ = (const bf16*)A.k_pages + ((size_t)pg_now * nkv + kvh) * AGAVE_PAGE * ksl * 32;
         const bf16* vb_ = (const bf16*)A.v_pages + ((size_t)pg_now * nkv + kvh) * (size_t)vd * AGAVE_PAGE;
         // What the page needs from memory is asked for before any of it is used (a wave's loads come back in the
         // order they left): the bias where it is read from memory, the value operands where the registers allow, then
@@ -380,7 +413,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
                 for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const int dist = pos[cb] - (pi * AGAVE_PAGE + 16 * kb + 4 * g + e);
+                        const int dist = pos[cb] - (pi * AGAVE_PAGE + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + e);
                         bv[cb][kb][e] = bias_row[dist < 0 ? 0 : (dist < A.bias_len ? dist : A.bias_len - 1)];
                     }
         }
@@ -389,26 +422,22 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
             for (int nb = 0; nb < VB; ++nb) {
                 // (a block past the value size reads the first block again and is not used)
-                const bf16* vr = vb_ + (size_t)((16 * nb < vd ? 16 * nb : 0) + c) * AGAVE_PAGE + 4 * g;
+                const bf16* vr = vb_ + ((size_t)(16 * nb < vd ? nb : 0) * 128 + lane) * 8;
 #pragma unroll
-                for (int h2 = 0; h2 < 2; ++h2) {
-                    const uint2 a0 = *reinterpret_cast<const uint2*>(vr + 32 * h2);
-                    const uint2 a1 = *reinterpret_cast<const uint2*>(vr + 32 * h2 + 16);
-                    va[V_AHEAD ? nb : 0][h2].u = make_uint4(a0.x, a0.y, a1.x, a1.y);
-                }
+                for (int h2 = 0; h2 < 2; ++h2) va[V_AHEAD ? nb : 0][h2].u = *reinterpret_cast<const uint4*>(vr + 512 * h2);
             }
         }
         // scores of the page's four key blocks
         f32x4_t s[NC][4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
-            const bf16* kr = kb_ + (size_t)(16 * kb + c) * hd + 8 * g;
+            // (a whole operand in one load of a kilobyte; steps past the head's end read step 0 again and are emptied)
+            const bf16* kr = kb_ + ((size_t)kb * ksl * 64 + lane) * 8;
             frag16 kf[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bool in = 32 * ks + 8 * g < hd;
-                const uint4 got = *reinterpret_cast<const uint4*>(kr + (in ? 32 * ks : -8 * g));
-                kf[ks].u = in ? got : make_uint4(0, 0, 0, 0);
+                const uint4 got = *reinterpret_cast<const uint4*>(kr + (ks < ksl ? ks * 512 : 0));
+                kf[ks].u = ks < ksl ? got : make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
             for (int cb = 0; cb < NC; ++cb) {
@@ -427,7 +456,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
             for (int kb = 0; kb < 4; ++kb) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int j = pi * AGAVE_PAGE + 16 * kb + 4 * g + e;
+                    const int j = pi * AGAVE_PAGE + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + e;
                     const int dist = pos[cb] - j;
                     const bool see = valid[cb] && dist >= 0 && (W == 0 || dist < W || j < keep);
                     float v = s[cb][kb][e] * A.scale;
@@ -477,13 +506,9 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
                     vf[0] = va[V_AHEAD ? nb : 0][0];
                     vf[1] = va[V_AHEAD ? nb : 0][1];
                 } else {
-                    const bf16* vr = vb_ + (size_t)(16 * nb + c) * AGAVE_PAGE + 4 * g;
+                    const bf16* vr = vb_ + ((size_t)nb * 128 + lane) * 8;
 #pragma unroll
-                    for (int h2 = 0; h2 < 2; ++h2) {
-                        const uint2 a0 = *reinterpret_cast<const uint2*>(vr + 32 * h2);
-                        const uint2 a1 = *reinterpret_cast<const uint2*>(vr + 32 * h2 + 16);
-                        vf[h2].u = make_uint4(a0.x, a0.y, a1.x, a1.y);
-                    }
+                    for (int h2 = 0; h2 < 2; ++h2) vf[h2].u = *reinterpret_cast<const uint4*>(vr + 512 * h2);
                 }
 #pragma unroll
                 for (int cb = 0; cb < NC; ++cb) {
@@ -513,7 +538,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
             for (int nb = 0; nb < VB; ++nb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) mine[32 + (16 * nb + 4 * g + e) * 16 + c] = o[0][nb][e];
+                for (int e = 0; e < 4; ++e) mine[32 + (16 * nb + 4 * g + (e ^ (g & 1))) * 16 + c] = o[0][nb][e];     // (odd lane groups swap neighbours: no two lanes of a half wave share a bank)
         }
         __syncthreads();
         if (w > 0) return;
@@ -528,7 +553,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
             for (int nb = 0; nb < VB; ++nb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[0][nb][e] = o[0][nb][e] * a1 + other[32 + (16 * nb + 4 * g + e) * 16 + c] * a2;
+                for (int e = 0; e < 4; ++e) o[0][nb][e] = o[0][nb][e] * a1 + other[32 + (16 * nb + 4 * g + (e ^ (g & 1))) * 16 + c] * a2;
         }
     }
 #pragma unroll
@@ -589,7 +614,7 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
                                       int window, int keep_first, int bias_mode, const float* bias, int bias_len,
                                       const float* sink, hipStream_t stream) {
     BiasedArgs A{q, ldq, out, ldo, gate, ldg, k_pages, v_pages, table, width, base, head, n_pages, tok_seq, tok_pos,
-                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink};
+                 nh, nkv, hd, vd, scale, window, keep_first, bias_mode, bias, bias_len, sink, 1};
     if (check_biased(A, N)) return -1;
     AGAVE_CHECK(agave_attn_biased_mfma_ok(hd, vd, (int)(ldq % 8), (int)(ldo % 4), (int)(ldg % 4)),
                 "attn_biased_mfma: head sizes %d / %d or row strides that the matrix-core kernel does not take", hd, vd);

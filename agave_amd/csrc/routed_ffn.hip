@@ -118,8 +118,10 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
                                                           const float* __restrict__ correction, int N, int K, int R, int groups,
                                                           int keep, int top, float scale, int* __restrict__ choice,
                                                           float* __restrict__ weight) {
-    extern __shared__ float zs[];                      // [ROUTE_ROWS][R]
+    extern __shared__ float zs[];                      // [ROUTE_ROWS][R], then the corrections [R]
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    float* corr = zs + ROUTE_ROWS * R;                 // (read many times by the one thread that chooses: from LDS, not memory)
+    for (int e = threadIdx.x; e < R; e += blockDim.x) corr[e] = correction ? correction[e] : 0.f;
     const int t0 = blockIdx.x * ROUTE_ROWS;
     const int rows = min(ROUTE_ROWS, N - t0);
     for (int r = w; r < R; r += nw) {
@@ -158,54 +160,63 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
         }
     }
     __syncthreads();
-    const int i = threadIdx.x;
-    if (i >= rows) return;
-    float* sr = zs + (size_t)i * R;
-    const int t = t0 + i;
-    float mx = -INFINITY;
-    for (int e = 0; e < R; ++e) mx = fmaxf(mx, sr[e]);
-    float sum = 0.f;
-    for (int e = 0; e < R; ++e) {
-        const float v = expf(sr[e] - mx);
-        sr[e] = v;
-        sum += v;
-    }
-    const float inv = 1.0f / sum;
-    for (int e = 0; e < R; ++e) sr[e] *= inv;
+    // the choice: a wave per token, the lanes along the outputs
     const int gs = R / groups;
-    unsigned long long open = ~0ull;
-    if (keep < groups) {
-        open = 0ull;
-        for (int r = 0; r < keep; ++r) {
-            int best = -1;
+    for (int i = w; i < rows; i += nw) {
+        float* sr = zs + (size_t)i * R;
+        const int t = t0 + i;
+        float mx = -INFINITY;
+        for (int e = lane; e < R; e += 64) mx = fmaxf(mx, sr[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < R; e += 64) {
+            const float v = expf(sr[e] - mx);
+            sr[e] = v;
+            sum += v;
+        }
+        const float inv = 1.0f / wave_sum(sum);
+        for (int e = lane; e < R; e += 64) sr[e] *= inv;
+        // the groups that stay open: lane g holds group g's score (at most 64 groups)
+        unsigned long long open = ~0ull;
+        if (keep < groups) {
+            float gv = -INFINITY;
+            if (lane < groups)
+                for (int e = lane * gs; e < (lane + 1) * gs; ++e) gv = fmaxf(gv, sr[e] + corr[e]);
+            open = 0ull;
+            for (int r = 0; r < keep; ++r) {
+                const float cand = (lane < groups && !((open >> lane) & 1ull)) ? gv : -INFINITY;
+                const float best_v = wave_max(cand);
+                // the lowest group among equals
+                const float first = wave_max((lane < groups && !((open >> lane) & 1ull) && cand == best_v) ? -(float)lane : -INFINITY);
+                open |= 1ull << (int)(-first);
+            }
+        }
+        // the `top` best of what is open; what was chosen is marked in the row's sign (s >= 0)
+        for (int r = 0; r < top; ++r) {
             float best_v = -INFINITY;
-            for (int g = 0; g < groups; ++g) {
-                if ((open >> g) & 1ull) continue;
-                float gv = -INFINITY;
-                for (int e = g * gs; e < (g + 1) * gs; ++e) gv = fmaxf(gv, sr[e] + (correction ? correction[e] : 0.f));
-                if (best < 0 || gv > best_v) {
-                    best = g;
-                    best_v = gv;
+            int best = -1;
+            for (int e = lane; e < R; e += 64) {
+                const float se = sr[e];
+                if (se < 0.f || !((open >> (e / gs)) & 1ull)) continue;
+                const float c = se + corr[e];
+                if (best < 0 || c > best_v) {          // (a lane's outputs come in rising order: the first of equals stays)
+                    best = e;
+                    best_v = c;
                 }
             }
-            open |= 1ull << best;
-        }
-    }
-    for (int r = 0; r < top; ++r) {
-        int best = -1;
-        float best_v = -INFINITY;
-        for (int e = 0; e < R; ++e) {
-            const float se = sr[e];
-            if (se < 0.f || !((open >> (e / gs)) & 1ull)) continue;
-            const float c = se + (correction ? correction[e] : 0.f);
-            if (best < 0 || c > best_v) {
-                best = e;
-                best_v = c;
+            const float top_v = wave_max(best >= 0 ? best_v : -INFINITY);
+            const int chosen = (int)(-wave_max((best >= 0 && best_v == top_v) ? -(float)best : -INFINITY));
+            // (top <= open outputs is checked on the host, so some lane has a candidate)
+            const float s_chosen = sr[chosen];
+            if (lane == 0) {
+                choice[(size_t)t * top + r] = chosen;
+                weight[(size_t)t * top + r] = s_chosen * scale;
+                sr[chosen] = -1.0f - s_chosen;
             }
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
-        choice[(size_t)t * top + r] = best;
-        weight[(size_t)t * top + r] = sr[best] * scale;
-        sr[best] = -1.0f - sr[best];
     }
 }
 
@@ -219,7 +230,7 @@ extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float*
     AGAVE_CHECK(x && router && choice && weight && ldx >= K, "route_rows: bad buffers");
     if (N == 0) return 0;
     const int blocks = (N + ROUTE_ROWS - 1) / ROUTE_ROWS;
-    const size_t lds = (size_t)ROUTE_ROWS * R * sizeof(float);
+    const size_t lds = (size_t)(ROUTE_ROWS + 1) * R * sizeof(float);
     const int threads = blocks < 128 ? 1024 : 256;
     const bool wide = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 32) == 0 && ((uintptr_t)router % 32) == 0;
     if (dtype == AGAVE_F32) {

@@ -18,9 +18,9 @@ LIBRARY = "attention_biased"
 BIAS_NONE, BIAS_SLOPES, BIAS_TABLE = 0, 1, 2
 
 kernels.register_signatures(LIBRARY, {
-    "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P],
+    "agave_kv_append_rows": [_I, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "agave_attn_biased_plain": [_I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F,
-                                _I, _I, _I, _P, _I, _P, _P],
+                                _I, _I, _I, _P, _I, _P, _I, _P],
     "agave_attn_biased_mfma_ok": [_I, _I, _I, _I, _I],
     "agave_attn_biased_mfma": [_P, _L, _P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
                                _F, _I, _I, _I, _P, _I, _P, _P],
@@ -31,9 +31,13 @@ def _lib():
     return kernels.lib(LIBRARY)
 
 
-def _check_row_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, vd: int, dtype: torch.dtype) -> int:
-    if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd) or not k_pages.is_contiguous():
-        raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd}], got {tuple(k_pages.shape)}")
+def _check_row_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, vd: int, dtype: torch.dtype,
+                     packed: bool = False) -> int:
+    if packed and (dtype != torch.bfloat16 or hd % 8 or vd % 16 or hd > 256 or vd > 256):
+        raise ValueError("pages in operand order hold bfloat16, keys in steps of 8 and values in steps of 16, up to 256")
+    hd_k = (hd + 31) // 32 * 32 if packed else hd       # operands are whole steps of 32 along the head
+    if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd_k) or not k_pages.is_contiguous():
+        raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd_k}], got {tuple(k_pages.shape)}")
     if v_pages.dim() != 4 or tuple(v_pages.shape[1:]) != (nkv, vd, 64) or not v_pages.is_contiguous():
         raise ValueError(f"V pages must be contiguous [pages, {nkv}, {vd}, 64], got {tuple(v_pages.shape)}")
     if k_pages.shape[0] != v_pages.shape[0] or k_pages.dtype != dtype or v_pages.dtype != dtype:
@@ -49,30 +53,33 @@ def _check_table(table: torch.Tensor, base: torch.Tensor, head: int, keep_first:
 
 
 def kv_append_rows(k: torch.Tensor, v: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, table: torch.Tensor,
-                   base: torch.Tensor, head: int, step, n_kv: int, head_dim: int, v_head_dim: int) -> None:
-    """The step's key and value rows into their places in the cache pages (row by row, as they are)."""
+                   base: torch.Tensor, head: int, step, n_kv: int, head_dim: int, v_head_dim: int, packed: bool = False) -> None:
+    """The step's key and value rows into their places in the cache pages: keys row by row and values transposed
+    inside a page, or (``packed``) both in the order the matrix-core kernel reads its operands."""
     _dev(k, v, k_pages, v_pages, table, base)
     n = step.n_tokens
     ldk, ldv = _rows(k, "k"), _rows(v, "v")
     if k.shape != (n, n_kv * head_dim) or v.shape != (n, n_kv * v_head_dim) or k.dtype != v.dtype:
         raise ValueError(f"k and v must be [{n}, {n_kv * head_dim}] and [{n}, {n_kv * v_head_dim}] of one dtype")
-    n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, k.dtype)
+    n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, k.dtype, packed)
     width = _check_table(table, base, head, 0)
     library.call(_lib(), "agave_kv_append_rows", dt(k), ptr(k), ldk, ptr(v), ldv, ptr(k_pages), ptr(v_pages), ptr(table),
                  width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n, n_kv, head_dim, v_head_dim,
-                 stream())
+                 1 if packed else 0, stream())
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torch.Tensor,
               v_pages: torch.Tensor, table: torch.Tensor, base: torch.Tensor, head: int, step, n_heads: int, n_kv: int,
               head_dim: int, v_head_dim: int, scale: float, window: Optional[int], keep_first: int, bias_mode: int,
-              bias: Optional[torch.Tensor], sink: Optional[torch.Tensor], force_plain: bool = False) -> None:
+              bias: Optional[torch.Tensor], sink: Optional[torch.Tensor], packed: bool = False,
+              force_plain: bool = False) -> None:
     """out[t, h] = sum_j w_j v_j with w = softmax_j(scale q.k_j + bias(h, p - j)) over the keys that token t at
     position p sees (j <= p and (p - j < window or j < keep_first)), the sink's exp(sink_h) added to the
     denominator, times sigmoid(gate[t, h]) element by element.  ``bias``: slopes [heads] (``BIAS_SLOPES``:
     the bias is -slope_h (p - j)) or a table [heads, distances] (``BIAS_TABLE``: distances beyond the table take
-    its last column).  bfloat16 rows with a key size that is a multiple of 8 and a value size that is a multiple of 16
-    (both up to 256) run on the matrix cores, everything else (and everything with ``force_plain``) on the plain kernel."""
+    its last column).  Pages in operand order (``packed``: bfloat16, a key size that is a multiple of 8 and a value size
+    that is a multiple of 16, both up to 256) run on the matrix cores, everything else (and everything with
+    ``force_plain``) on the plain kernel, which reads either order."""
     _dev(q, out, gate, k_pages, v_pages, table, base, bias, sink)
     n = step.n_tokens
     ldq, ldo = _rows(q, "q"), _rows(out, "out")
@@ -83,7 +90,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
         ldg = _rows(gate, "gate")
         if gate.shape != out.shape or gate.dtype != q.dtype:
             raise ValueError("attention: the gate must have the output's shape and dtype")
-    n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, q.dtype)
+    n_pages = _check_row_pages(k_pages, v_pages, n_kv, head_dim, v_head_dim, q.dtype, packed)
     width = _check_table(table, base, head, keep_first)
     bias_len = 0
     if bias_mode == BIAS_SLOPES:
@@ -95,7 +102,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
     elif bias_mode != BIAS_NONE:
         raise ValueError(f"attention: unknown bias mode {bias_mode}")
     _f32vec(sink, "sink", n_heads)
-    if q.dtype == torch.bfloat16 and not force_plain and _lib().agave_attn_biased_mfma_ok(head_dim, v_head_dim, ldq, ldo, ldg) \
+    if packed and not force_plain and _lib().agave_attn_biased_mfma_ok(head_dim, v_head_dim, ldq, ldo, ldg) \
             and q.data_ptr() % 16 == 0 and out.data_ptr() % 8 == 0:
         # the matrix cores: 16 rows of a head a wave in a step of many rows, a row's heads of one key head in a
         # step of one row a sequence
@@ -110,4 +117,4 @@ def attention(q: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor], 
     library.call(_lib(), "agave_attn_biased_plain", dt(q), ptr(q), ldq, ptr(out), ldo, ptr(gate), ldg, ptr(k_pages),
                  ptr(v_pages), ptr(table), width, ptr(base), head, n_pages, ptr(step.tok_seq), ptr(step.tok_pos), n,
                  n_heads, n_kv, head_dim, v_head_dim, float(scale), int(window or 0), int(keep_first), bias_mode,
-                 ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), stream())
+                 ptr(bias) if bias_mode != BIAS_NONE else None, bias_len, ptr(sink), 1 if packed else 0, stream())

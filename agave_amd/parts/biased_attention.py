@@ -129,7 +129,7 @@ class BiasedAttention:
             raise ValueError("biased attention: a mixer with key and value projections appends to its memory, one "
                              "without reads another's; the run order says otherwise")
         group = step.cache.group_of_memory[memory]
-        k_pages, v_pages, _ = step.cache.pages_of(memory)
+        k_pages, v_pages, packed = step.cache.pages_of(memory)
         table, base = step.tables[group]
         head = step.cache.group_keys[group].kept_pages
         proj = self.proj.forward(x, tag="qkvg")
@@ -138,12 +138,12 @@ class BiasedAttention:
         at = 1
         if self.own_kv:
             ops.kv_append_rows(cols[1], cols[2], k_pages, v_pages, table, base, head, step, s.n_kv_heads, s.head_dim,
-                               s.v_head_dim)
+                               s.v_head_dim, packed)
             at = 3
         gate = cols[at] if s.gate_proj else None
         ctx = ws.get("attn_ctx", n, self.ctx, x.dtype)
         ops.attention(q, ctx, gate, k_pages, v_pages, table, base, head, step, s.n_heads, s.n_kv_heads, s.head_dim,
-                      s.v_head_dim, s.scale, s.window, s.keep_first, self.bias_mode, self.bias, self.sink)
+                      s.v_head_dim, s.scale, s.window, s.keep_first, self.bias_mode, self.bias, self.sink, packed)
         return self.o.forward(ctx, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream
 
 

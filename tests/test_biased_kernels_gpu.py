@@ -95,14 +95,14 @@ class Case:
         sink = self.sink.to(DEV) if self.sink is not None else None
         for lo, hi in ranges:
             step = planner.plan([slot], [[0] * (hi - lo)], "all")
-            kp, vp, _ = cache.pages_of(0)
+            kp, vp, packed = cache.pages_of(0)
             table, base = step.tables[0]
             dev = lambda t: t[lo:hi].reshape(hi - lo, -1).to(dtype).to(DEV).contiguous()
-            A.kv_append_rows(dev(self.k), dev(self.v), kp, vp, table, base, head, step, self.G, self.d, self.vd)
+            A.kv_append_rows(dev(self.k), dev(self.v), kp, vp, table, base, head, step, self.G, self.d, self.vd, packed)
             out = torch.empty(hi - lo, self.H * self.vd, dtype=dtype, device=DEV)
             A.attention(dev(self.q), out, dev(self.gate) if self.gate is not None else None, kp, vp, table, base, head, step,
                         self.H, self.G, self.d, self.vd, self.scale, self.window, self.keep, self.mode, self.bias, sink,
-                        force_plain=self.force_plain)
+                        packed, force_plain=self.force_plain)
             planner.commit(step)
             got[lo:hi] = out.float().cpu()
         if own:
@@ -167,14 +167,14 @@ def test_a_batch_against_each_alone_and_slots_and_pages_used_again(dtype):
         while live:
             n_new = [firsts[i] if first else 1 for i in live]
             step = planner.plan([slots[i] for i in live], [[0] * n for n in n_new], "all")
-            kp, vp, _ = cache.pages_of(0)
+            kp, vp, packed = cache.pages_of(0)
             table, base = step.tables[0]
             cat = lambda name: torch.cat([getattr(cases[i], name)[used[i]:used[i] + n].reshape(n, -1)
                                           for i, n in zip(live, n_new)]).to(dtype).to(DEV).contiguous()
-            A.kv_append_rows(cat("k"), cat("v"), kp, vp, table, base, key.kept_pages, step, 2, 16, 24)
+            A.kv_append_rows(cat("k"), cat("v"), kp, vp, table, base, key.kept_pages, step, 2, 16, 24, packed)
             out = torch.empty(sum(n_new), 4 * 24, dtype=dtype, device=DEV)
             A.attention(cat("q"), out, cat("gate"), kp, vp, table, base, key.kept_pages, step, 4, 2, 16, 24, cases[0].scale,
-                        50, 4, cases[0].mode, cases[0].bias, None)
+                        50, 4, cases[0].mode, cases[0].bias, None, packed)
             planner.commit(step)
             at = 0
             for i, n in zip(live, n_new):
