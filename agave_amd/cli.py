@@ -76,7 +76,7 @@ def model_info(engine) -> dict:
             "bos_token_id": s.bos_token_id, "eos_token_ids": list(s.eos_token_ids),
             "weight_bytes": engine.model.weight_bytes(), "cache_bytes": engine.cache.bytes(),
             "cache_groups": [{"window": k.window, "chunk": k.chunk, "n_kv_heads": k.n_kv_heads, "head_dim": k.head_dim,
-                              "v_head_dim": k.v_head_dim or k.head_dim, "layout": k.layout}
+                              "v_head_dim": k.v_head_dim or k.head_dim, "layout": k.layout, "keep_first": k.keep_first}
                              for k in engine.cache.group_keys],
             "state_bytes": sum(t.numel() * t.element_size() for t in engine.cache._state_tensors())}
 

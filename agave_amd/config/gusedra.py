@@ -113,7 +113,7 @@ class GusedraConfig:
             bias_max = kv_from = None
             if kind == "attention_2":
                 bias_max = _int(m, "bias_max", mw)
-            elif m.get("kv_from") is not None:
+            if m.get("kv_from") is not None:
                 kv_from = _int(m, "kv_from", mw, least=0)
             mixer = GusedraMixer(kind, heads, kv_heads, _int(m, "dim", mw), _int(m, "vdim", mw), _num(m, "scale", mw),
                                  window, keep_first, bias_max, kv_from)

@@ -452,7 +452,7 @@ template <int MI, int NJ, bool GATED>
 __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __restrict__ x, long ldx, const int* __restrict__ sorted_pair,
                                                                   const int* __restrict__ tile_expert, const bf16* __restrict__ w0,
                                                                   const bf16* __restrict__ w1, void* __restrict__ out_, int top,
-                                                                  int n_out, int K, int act) {
+                                                                  int n_out, int K, int act, int wpacked) {
     const int e = tile_expert[blockIdx.x];
     if (e < 0) return;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -479,8 +479,12 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
     for (int j = 0; j < NJ; ++j) {
         int col = col0 + 16 * j + c;
         if (col >= n_out) col = n_out - 1;
-        b0[j] = w0 + ((size_t)e * n_out + col) * K + 8 * g;
-        b1[j] = GATED ? w1 + ((size_t)e * n_out + col) * K + 8 * g : nullptr;
+        // (wpacked: W[e] in tiles of 16 rows x 32 columns, each the 64 lanes' operands in a row, a row block's tiles one
+        // after another: a whole operand is one load of a kilobyte)
+        const size_t at0 = wpacked ? (((size_t)e * (n_out / 16) + col / 16) * (K / 32) * 64 + lane) * 8
+                                   : ((size_t)e * n_out + col) * K + 8 * g;
+        b0[j] = w0 + at0;
+        b1[j] = GATED ? w1 + at0 : nullptr;
     }
     f32x4_t acc0[MI][NJ], acc1[MI][GATED ? NJ : 1];
 #pragma unroll
@@ -490,17 +494,44 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
             acc0[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             if (GATED) acc1[i][GATED ? j : 0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
-    for (int k0 = 0; k0 < K; k0 += 32) {
+    int k_done = 0;
+    if constexpr (MI == 1) {
+        // a tile of 16 rows streams its weights once and waits for memory, not for the matrix cores: the loads of
+        // eight steps are asked for before the first is used
+        constexpr int U = 8;
+        for (; k_done + 32 * U <= K; k_done += 32 * U) {
+            frag16 a[U], bw0[U][NJ], bw1[U][NJ];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int k0 = k_done + 32 * u;
+                a[u].u = *reinterpret_cast<const uint4*>(arow[0] + k0);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    bw0[u][j].u = *reinterpret_cast<const uint4*>(b0[j] + (wpacked ? k0 * 16 : k0));
+                    if (GATED) bw1[u][j].u = *reinterpret_cast<const uint4*>(b1[j] + (wpacked ? k0 * 16 : k0));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    acc0[0][j] = mfma_16x16x32(a[u], bw0[u][j], acc0[0][j]);
+                    if (GATED) acc1[0][GATED ? j : 0] = mfma_16x16x32(a[u], bw1[u][j], acc1[0][GATED ? j : 0]);
+                }
+        }
+    }
+    for (int k0 = k_done; k0 < K; k0 += 32) {
         // (loads without conditions, from inside the row; a lane past the row's end reads its start and is emptied)
         const bool in = k0 + 8 * g < K;
         const int at = in ? k0 : -8 * g;
+        const int bat = wpacked ? k0 * 16 : at;
         frag16 a[MI], bw0[NJ], bw1[NJ];
 #pragma unroll
         for (int i = 0; i < MI; ++i) a[i].u = *reinterpret_cast<const uint4*>(arow[i] + at);
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            bw0[j].u = *reinterpret_cast<const uint4*>(b0[j] + at);
-            if (GATED) bw1[j].u = *reinterpret_cast<const uint4*>(b1[j] + at);
+            bw0[j].u = *reinterpret_cast<const uint4*>(b0[j] + bat);
+            if (GATED) bw1[j].u = *reinterpret_cast<const uint4*>(b1[j] + bat);
         }
         if (!in) {
 #pragma unroll
@@ -538,7 +569,8 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
 // act_rows [cap, ff] bfloat16 and y [cap, hidden] float32 hold sorted rows (see route_sort)
 extern "C" int agave_routed_experts_mfma(const void* x, long ldx, const int* sorted_pair, const int* tile_expert, const void* wg,
                                          const void* wu, const void* wd, void* act_rows, float* y, int TM, int max_tiles, int top,
-                                         int E, int ff, int hidden, int act, hipStream_t stream) {
+                                         int E, int ff, int hidden, int act, int wpacked, hipStream_t stream) {
+    AGAVE_CHECK(!wpacked || (ff % 32 == 0 && hidden % 32 == 0), "routed_experts_mfma: weights in tile order need sizes that are multiples of 32");
     AGAVE_CHECK(max_tiles > 0 && top > 0 && E > 0 && ff > 0 && hidden > 0 && (TM == 16 || TM == 64), "routed_experts_mfma: bad sizes");
     AGAVE_CHECK(act >= 0 && act < 4, "routed_experts_mfma: unknown activation %d", act);
     AGAVE_CHECK(hidden % 8 == 0 && ff % 8 == 0 && ldx % 8 == 0, "routed_experts_mfma: sizes must be multiples of 8 (hidden %d, ff %d)", hidden, ff);
@@ -546,20 +578,20 @@ extern "C" int agave_routed_experts_mfma(const void* x, long ldx, const int* sor
     AGAVE_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wg % 16) == 0 && ((uintptr_t)wu % 16) == 0 && ((uintptr_t)wd % 16) == 0 &&
                 ((uintptr_t)act_rows % 16) == 0, "routed_experts_mfma: buffers must be aligned to 16 bytes");
     // tiles of 64 rows take 64 columns a wave (an operand that was loaded serves more multiplications), tiles of
-    // 16 rows, which stream their weights once, 32
-    const int cols = TM == 64 ? 256 : 128;
+    // 16 rows, which stream their weights once, 16 (more workgroups, each with many loads in flight)
+    const int cols = TM == 64 ? 256 : 64;
     const dim3 g1(max_tiles, (ff + cols - 1) / cols), g2(max_tiles, (hidden + cols - 1) / cols);
     AGAVE_CHECK(g1.y <= 65535 && g2.y <= 65535, "routed_experts_mfma: too many columns for the grid");
     if (TM == 64) {
         routed_product_mfma_kernel<4, 4, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
-                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act);
+                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act, wpacked);
         routed_product_mfma_kernel<4, 4, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
-                                                                     nullptr, y, top, hidden, ff, act);
+                                                                     nullptr, y, top, hidden, ff, act, wpacked);
     } else {
-        routed_product_mfma_kernel<1, 2, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
-                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act);
-        routed_product_mfma_kernel<1, 2, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
-                                                                     nullptr, y, top, hidden, ff, act);
+        routed_product_mfma_kernel<1, 1, true><<<g1, 256, 0, stream>>>((const bf16*)x, ldx, sorted_pair, tile_expert, (const bf16*)wg,
+                                                                    (const bf16*)wu, act_rows, top, ff, hidden, act, wpacked);
+        routed_product_mfma_kernel<1, 1, false><<<g2, 256, 0, stream>>>((const bf16*)act_rows, ff, sorted_pair, tile_expert, (const bf16*)wd,
+                                                                     nullptr, y, top, hidden, ff, act, wpacked);
     }
     AGAVE_LAUNCH_CHECK("routed_experts_mfma");
     return 0;

@@ -16,7 +16,7 @@ kernels.register_signatures(LIBRARY, {
     "agave_routed_experts_plain": [_I, _P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "agave_route_rows": [_I, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P, _P],
     "agave_route_sort": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
-    "agave_routed_experts_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "agave_routed_experts_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "agave_routed_combine": [_I, _P, _P, _P, _P, _P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _P],
 })
 
@@ -118,9 +118,11 @@ def route_sort(choice: torch.Tensor, n_experts: int, tm: int, tiles: int, place:
 
 
 def experts_mfma(x: torch.Tensor, sorted_pair: torch.Tensor, tile_expert: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
-                 w_down: torch.Tensor, act_rows: torch.Tensor, y: torch.Tensor, tm: int, tiles: int, top: int, activation: int) -> None:
+                 w_down: torch.Tensor, act_rows: torch.Tensor, y: torch.Tensor, tm: int, tiles: int, top: int, activation: int,
+                 tile_order: bool = False) -> None:
     """The experts' products over the sorted rows on the matrix cores: ``act_rows`` [tiles * tm, ff] bfloat16 and
-    ``y`` [tiles * tm, hidden] float32 receive sorted rows (padding rows hold nothing of use)."""
+    ``y`` [tiles * tm, hidden] float32 receive sorted rows (padding rows hold nothing of use).  ``tile_order``: the
+    weights were rearranged by :func:`pack_expert_weights` (same shapes)."""
     _dev(x, sorted_pair, tile_expert, w_gate, w_up, w_down, act_rows, y)
     n, hidden = x.shape
     e, ff, k = w_gate.shape
@@ -139,7 +141,8 @@ def experts_mfma(x: torch.Tensor, sorted_pair: torch.Tensor, tile_expert: torch.
     _i32(sorted_pair, "sorted_pair", cap)
     _i32(tile_expert, "tile_expert", tiles)
     library.call(_lib(), "agave_routed_experts_mfma", ptr(x), x.stride(0), ptr(sorted_pair), ptr(tile_expert), ptr(w_gate),
-                 ptr(w_up), ptr(w_down), ptr(act_rows), ptr(y), tm, tiles, top, e, ff, hidden, activation, stream())
+                 ptr(w_up), ptr(w_down), ptr(act_rows), ptr(y), tm, tiles, top, e, ff, hidden, activation,
+                 1 if tile_order else 0, stream())
 
 
 def route_rows(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
@@ -158,3 +161,14 @@ def route_rows(x: torch.Tensor, router: torch.Tensor, correction: Optional[torch
         raise ValueError("route_rows: weight must be contiguous float32 [N, top]")
     library.call(_lib(), "agave_route_rows", dt(x), ptr(x), ldx, ptr(router), ptr(correction), n, k, r, groups, keep, top,
                  float(scale), ptr(choice), ptr(weight), stream())
+
+
+def pack_expert_weights(w: torch.Tensor) -> torch.Tensor:
+    """[E, N, K] (N a multiple of 16, K of 32) rearranged into the matrix cores' operand tiles: tiles of 16 rows by 32
+    columns, each stored as its 64 lanes' 16 bytes one after another (lane c + 16 g holds row c, columns 8 g .. 8 g + 7),
+    a row block's tiles along K following each other.  Same shape and bytes; only :func:`experts_mfma` reads it."""
+    e, n, k = w.shape
+    if n % 16 or k % 32:
+        raise ValueError("pack_expert_weights: rows must be a multiple of 16 and columns of 32")
+    t = w.view(e, n // 16, 16, k // 32, 4, 8).permute(0, 1, 3, 4, 2, 5).contiguous()      # [E, nb, kb, g, c, 8]
+    return t.view(e, n, k)

@@ -51,8 +51,12 @@ class RoutedFfn:
         def stack(which: str) -> torch.Tensor:
             mats = [weights.get(f"{s.expert_prefix}{i}.{which}") for i in range(s.n_experts)]
             return torch.stack([m.to(env.dtype) for m in mats]).contiguous().to(dev)     # [experts, out, in]
+        # bfloat16 experts whose sizes are multiples of 32 are kept in the matrix cores' tile order (only that copy)
+        self.tile_order = bool(s.n_experts) and env.dtype == torch.bfloat16 and s.hidden % 32 == 0 and s.intermediate % 32 == 0
         if s.n_experts:
             self.w_gate, self.w_up, self.w_down = stack(s.gate_name), stack(s.up_name), stack(s.down_name)
+            if self.tile_order:
+                self.w_gate, self.w_up, self.w_down = (routed.pack_expert_weights(w) for w in (self.w_gate, self.w_up, self.w_down))
         else:
             self.w_gate = self.w_up = self.w_down = None
         self.shared = GatedFfn(s.shared, weights, env) if s.shared is not None else None
@@ -81,6 +85,8 @@ class RoutedFfn:
         # the router's 32-bit product and the choice in one kernel
         routed.route_rows(x, self.router, self.correction, s.groups, s.keep_groups, top, s.route_scale, choice, weight)
         y = place = None
+        if self.tile_order and not routed.mfma_ok(x, s.intermediate):
+            raise ValueError("routed feed-forward: its experts are kept in tile order, which takes aligned bfloat16 rows")
         if s.n_experts and self.w_gate.dtype == torch.bfloat16 and routed.mfma_ok(x, s.intermediate):
             # the pairs sorted by expert on the device, then the experts' products tile by tile on the matrix cores
             tm, tiles, cap = routed.tile_plan(n * top, s.n_experts)
@@ -91,7 +97,7 @@ class RoutedFfn:
             act_rows = ws.get("expert_act", cap, s.intermediate, x.dtype)
             y = ws.get("expert_rows", cap, s.hidden, torch.float32)
             routed.experts_mfma(x, sorted_pair, tile_expert, self.w_gate, self.w_up, self.w_down, act_rows, y, tm, tiles, top,
-                                self.act)
+                                self.act, tile_order=self.tile_order)
         elif s.n_experts:
             act_rows = ws.get("expert_act", n * top, s.intermediate, x.dtype)
             y = ws.get("expert_rows", n * top, s.hidden, torch.float32)

@@ -378,7 +378,7 @@ def test_route_groups_decide_before_the_experts():
 # ---------------------------------------------------------------- the experts and their sum
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("E, I, top, ff, hidden, n", [(5, 2, 3, 20, 40, 33), (3, 0, 1, 70, 24, 5), (8, 1, 8, 16, 72, 130), (0, 2, 2, 8, 16, 4),
-                                                    (6, 1, 2, 136, 200, 300), (4, 2, 3, 256, 128, 70)])
+                                                    (6, 1, 2, 136, 200, 300), (4, 2, 3, 256, 128, 70), (3, 1, 2, 96, 160, 200)])
 def test_experts_and_their_weighted_sum(dtype, E, I, top, ff, hidden, n):
     from agave_amd.ops import routed
     g = torch.Generator().manual_seed(E * 10 + top)
@@ -428,3 +428,9 @@ def test_experts_and_their_weighted_sum(dtype, E, I, top, ff, hidden, n):
             routed.combine(y2, place, choice.view(-1).to(DEV), weight.view(-1).to(DEV), d(x), d(shared), out2, top, E)
             err = (out2.float().cpu().to(F64) - want).abs().max()
             assert float(err) <= tol * float(want.abs().max()), f"tiles of {tm}: error {float(err):.3e}"
+            if ff % 32 == 0 and hidden % 32 == 0:          # the same with the weights in tile order
+                y3 = torch.full((tiles * tm, hidden), float("nan"), device=DEV)
+                routed.experts_mfma(d(x), sorted_pair, tile_expert, routed.pack_expert_weights(d(wg)), routed.pack_expert_weights(d(wu)),
+                                    routed.pack_expert_weights(d(wd)), act_rows, y3, tm, tiles, top, 1, tile_order=True)
+                real = (sorted_pair >= 0)
+                assert torch.equal(y3[real], y2[real]), "weights in tile order give other sums"
