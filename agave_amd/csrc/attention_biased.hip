@@ -288,7 +288,9 @@ struct MfmaMode {
     int table_in_lds;            // the bias table's row of this head is copied to LDS (many rows)
 };
 
-template <int KS, int VB, int NC>
+typedef __attribute__((address_space(3))) u32x4_t lds_u32x4;
+
+template <int KS, int VB, int NC, bool LDSP>
 __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, MfmaMode M) {
     extern __shared__ float lds_generic[];
     // (every LDS access goes through a pointer that says so: no pointer may end up chosen between the two memories)
@@ -304,6 +306,8 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
     int row[NC], pos[NC], head, b;
     bool valid[NC];
     int pmin, pmax;                                 // the wave's range of positions (the same in every lane)
+    int wg_first = 0, wg_last = 0;                  // the workgroup's (many rows)
+    bool wave_on = true;
     if (M.one_row) {
         row[0] = blockIdx.x;
         b = A.tok_seq[row[0]];
@@ -325,11 +329,12 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         head = blockIdx.z;
         if (M.table_in_lds) {                                   // (before any wave leaves: all of them meet at the barrier)
             const float* src = A.bias + (size_t)head * A.bias_len;
-            for (int i = threadIdx.x; i < A.bias_len; i += blockDim.x) lds[i] = src[i];
+            for (int i = threadIdx.x; i < A.bias_len; i += blockDim.x) lds[i] = src[i] * 1.4426950408889634f;
             __syncthreads();
         }
         const int wr0 = r0 + w * WROWS;
-        if (wr0 >= r1) return;                                  // this wave has no rows; no barrier follows in this mode
+        wave_on = wr0 < r1;
+        if (!LDSP && !wave_on) return;                          // this wave has no rows (with pages through LDS it still carries them)
 #pragma unroll
         for (int cb = 0; cb < NC; ++cb) {
             row[cb] = wr0 + 16 * cb + c;
@@ -337,8 +342,10 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
             if (!valid[cb]) row[cb] = r1 - 1;
             pos[cb] = A.tok_pos[row[cb]];
         }
-        pmin = A.tok_pos[wr0];
+        pmin = A.tok_pos[wave_on ? wr0 : r1 - 1];
         pmax = A.tok_pos[min(wr0 + WROWS, r1) - 1];
+        wg_first = A.tok_pos[r0];
+        wg_last = A.tok_pos[min(r0 + 4 * WROWS, r1) - 1];
     }
     const int kvh = head / per;
     const int ksl = (hd + 31) / 32;                 // steps along the head that the pages hold
@@ -349,9 +356,10 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
     const int n_pg = n_kept + pmax / AGAVE_PAGE - first_win + 1;
     const int pbase = A.base[b];
 
+    const float LOG2E = 1.4426950408889634f;
     const float* bias_row = nullptr;           // table of my head
-    float slope = 0.f;
-    if (A.bias_mode == 1) slope = A.bias[head];
+    const float scale2 = A.scale * LOG2E;
+    const float slope2 = A.bias_mode == 1 ? A.bias[head] * LOG2E : 0.f;
     if (A.bias_mode == 2) bias_row = A.bias + (size_t)head * A.bias_len;
 
     // Q as the B operand: lane holds Q[column c][32 ks + 8 g .. + 8]
@@ -378,7 +386,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         m[cb] = -INFINITY;
         l[cb] = 0.f;
         if (A.sink && (!M.one_row || w == 0)) {
-            m[cb] = A.sink[head];
+            m[cb] = A.sink[head] * LOG2E;
             l[cb] = g == 0 ? 1.f : 0.f;         // the lane groups' sums are added up at the end
         }
     }
@@ -391,16 +399,9 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
         const long pg = (col >= 0 && col < A.width) ? A.table[(size_t)b * A.width + col] : -1;
         return pg < A.n_pages ? pg : -1;
     };
-    int idx = M.one_row ? w : 0;
-    long pg = page_of(idx);
-    for (; idx < n_pg; idx += stride) {
-        const long pg_next = page_of(idx + stride);         // asked for now, used in the next turn
-        const long pg_now = pg;
-        pg = pg_next;
-        if (pg_now < 0) continue;
-        const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
-        const bf16* kb_ = (const bf16*)A.k_pages + ((size_t)pg_now * nkv + kvh) * AGAVE_PAGE * ksl * 32;
-        const bf16* vb_ = (const bf16*)A.v_pages + ((size_t)pg_now * nkv + kvh) * (size_t)vd * AGAVE_PAGE;
+    // One page: kt and vt hold its key and value operands, 64 lanes x 16 bytes each (tile (kb, ks) of the keys at
+    // kb ksl + ks, tile (nb, h) of the values at 2 nb + h), in memory or in LDS.
+    auto page = [&](int pi, auto kt, auto vt) {
         // What the page needs from memory is asked for before any of it is used (a wave's loads come back in the
         // order they left): the bias where it is read from memory, the value operands where the registers allow, then
         // the keys.
@@ -414,7 +415,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int dist = pos[cb] - (pi * AGAVE_PAGE + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + e);
-                        bv[cb][kb][e] = bias_row[dist < 0 ? 0 : (dist < A.bias_len ? dist : A.bias_len - 1)];
+                        bv[cb][kb][e] = bias_row[dist < 0 ? 0 : (dist < A.bias_len ? dist : A.bias_len - 1)] * LOG2E;
                     }
         }
         frag16 va[V_AHEAD ? VB : 1][2];
@@ -422,9 +423,8 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
             for (int nb = 0; nb < VB; ++nb) {
                 // (a block past the value size reads the first block again and is not used)
-                const bf16* vr = vb_ + ((size_t)(16 * nb < vd ? nb : 0) * 128 + lane) * 8;
 #pragma unroll
-                for (int h2 = 0; h2 < 2; ++h2) va[V_AHEAD ? nb : 0][h2].u = *reinterpret_cast<const uint4*>(vr + 512 * h2);
+                for (int h2 = 0; h2 < 2; ++h2) va[V_AHEAD ? nb : 0][h2].r = vt[((16 * nb < vd ? nb : 0) * 2 + h2) * 64 + lane];
             }
         }
         // scores of the page's four key blocks
@@ -432,12 +432,11 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
             // (a whole operand in one load of a kilobyte; steps past the head's end read step 0 again and are emptied)
-            const bf16* kr = kb_ + ((size_t)kb * ksl * 64 + lane) * 8;
             frag16 kf[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const uint4 got = *reinterpret_cast<const uint4*>(kr + (ks < ksl ? ks * 512 : 0));
-                kf[ks].u = ks < ksl ? got : make_uint4(0, 0, 0, 0);
+                const u32x4_t got = kt[(kb * ksl + (ks < ksl ? ks : 0)) * 64 + lane];
+                kf[ks].r = ks < ksl ? got : u32x4_t{0u, 0u, 0u, 0u};
             }
 #pragma unroll
             for (int cb = 0; cb < NC; ++cb) {
@@ -446,56 +445,72 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
                 for (int ks = 0; ks < KS; ++ks) s[cb][kb] = mfma_16x16x32(kf[ks], qf[cb][ks], s[cb][kb]);
             }
         }
-        // scale, bias, mask, softmax a column block at a time
+        // Scale, bias, mask and softmax, a column block at a time, in the base-2 domain (scale, slopes, table and
+        // sinks carry the factor log2(e), so an exponential is one instruction).  A page that every row of the wave
+        // sees whole (below the diagonal, inside the window or among the kept positions) needs no mask: most pages
+        // of a long sequence are such, and the mask is most of the arithmetic of a score.
         frag16 pf[NC][2];
         float alpha[NC];
+        const int j_last = pi * AGAVE_PAGE + AGAVE_PAGE - 1;
+        const bool whole = j_last <= pmin && (W == 0 || pmax - pi * AGAVE_PAGE < W || j_last < keep);
+        auto scores = [&](auto whole_tag, auto table_tag) {
+            constexpr bool WHOLE = decltype(whole_tag)::value != 0, TABLE = decltype(table_tag)::value != 0;
 #pragma unroll
-        for (int cb = 0; cb < NC; ++cb) {
-            float tile_max = -INFINITY;
+            for (int cb = 0; cb < NC; ++cb) {
+                float tile_max = -INFINITY;
+                const int d0 = pos[cb] - pi * AGAVE_PAGE - 8 * g;           // distance to the lane group's first key
+                const float t0 = -slope2 * (float)d0;
 #pragma unroll
-            for (int kb = 0; kb < 4; ++kb) {
+                for (int kb = 0; kb < 4; ++kb) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int j = pi * AGAVE_PAGE + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + e;
-                    const int dist = pos[cb] - j;
-                    const bool see = valid[cb] && dist >= 0 && (W == 0 || dist < W || j < keep);
-                    float v = s[cb][kb][e] * A.scale;
-                    if (A.bias_mode == 1) v -= slope * (float)dist;
-                    if (A.bias_mode == 2) {
-                        const int at = see ? (dist < A.bias_len ? dist : A.bias_len - 1) : 0;
-                        v += M.table_in_lds ? lds[at] : bv[cb][kb][e];
+                    for (int e = 0; e < 4; ++e) {
+                        const int off = 32 * (kb >> 1) + 4 * (kb & 1) + e;  // (a constant once the loops are unrolled)
+                        const int dist = d0 - off;
+                        float v = fmaf(s[cb][kb][e], scale2, fmaf(slope2, (float)off, t0));
+                        bool see = true;
+                        if (!WHOLE) see = valid[cb] && dist >= 0 && (W == 0 || dist < W || pos[cb] - dist < keep);
+                        if (TABLE) {
+                            int at = dist < A.bias_len ? dist : A.bias_len - 1;
+                            if (!WHOLE) at = see ? at : 0;
+                            v += M.table_in_lds ? lds[at] : bv[cb][kb][e];
+                        }
+                        if (!WHOLE) v = see ? v : -INFINITY;
+                        s[cb][kb][e] = v;
+                        tile_max = fmaxf(tile_max, v);
                     }
-                    v = see ? v : -INFINITY;
-                    s[cb][kb][e] = v;
-                    tile_max = fmaxf(tile_max, v);
                 }
-            }
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-            const float m_new = fmaxf(m[cb], tile_max);
-            // (a column that sees nothing of this page and has seen nothing before keeps m = -inf; its p are 0)
-            const float ref = m_new == -INFINITY ? 0.f : m_new;
-            alpha[cb] = m[cb] == -INFINITY ? 0.f : __expf(m[cb] - ref);
-            float sum = 0.f;
+                tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+                tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+                const float m_new = fmaxf(m[cb], tile_max);
+                // (a column that sees nothing of this page and has seen nothing before keeps m = -inf; its p are 0)
+                const float ref = m_new == -INFINITY ? 0.f : m_new;
+                alpha[cb] = m[cb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[cb] - ref);
+                float sum = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 4; ++kb) {
-                float p[4];
+                for (int kb = 0; kb < 4; ++kb) {
+                    float p[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    p[e] = __expf(s[cb][kb][e] - ref);          // exp(-inf) = 0 for what is not seen
-                    sum += p[e];
+                    for (int e = 0; e < 4; ++e) {
+                        p[e] = __builtin_amdgcn_exp2f(s[cb][kb][e] - ref);      // 2^(-inf) = 0 for what is not seen
+                        sum += p[e];
+                    }
+                    const uint32_t lo2 = f32x2_to_bf16x2(p[0], p[1]), hi2 = f32x2_to_bf16x2(p[2], p[3]);
+                    if (kb & 1) {
+                        pf[cb][kb >> 1].r[2] = lo2;
+                        pf[cb][kb >> 1].r[3] = hi2;
+                    } else {
+                        pf[cb][kb >> 1].r[0] = lo2;
+                        pf[cb][kb >> 1].r[1] = hi2;
+                    }
                 }
-                const uint32_t lo2 = f32x2_to_bf16x2(p[0], p[1]), hi2 = f32x2_to_bf16x2(p[2], p[3]);
-                if (kb & 1) {
-                    pf[cb][kb >> 1].r[2] = lo2;
-                    pf[cb][kb >> 1].r[3] = hi2;
-                } else {
-                    pf[cb][kb >> 1].r[0] = lo2;
-                    pf[cb][kb >> 1].r[1] = hi2;
-                }
+                l[cb] = l[cb] * alpha[cb] + sum;
+                m[cb] = m_new;
             }
-            l[cb] = l[cb] * alpha[cb] + sum;
-            m[cb] = m_new;
+        };
+        if (A.bias_mode == 2) {
+            if (whole) scores(IntC<1>{}, IntC<1>{}); else scores(IntC<0>{}, IntC<1>{});
+        } else {
+            if (whole) scores(IntC<1>{}, IntC<0>{}); else scores(IntC<0>{}, IntC<0>{});
         }
         // O^T = O^T alpha + V^T P^T
 #pragma unroll
@@ -506,9 +521,8 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
                     vf[0] = va[V_AHEAD ? nb : 0][0];
                     vf[1] = va[V_AHEAD ? nb : 0][1];
                 } else {
-                    const bf16* vr = vb_ + ((size_t)nb * 128 + lane) * 8;
 #pragma unroll
-                    for (int h2 = 0; h2 < 2; ++h2) vf[h2].u = *reinterpret_cast<const uint4*>(vr + 512 * h2);
+                    for (int h2 = 0; h2 < 2; ++h2) vf[h2].r = vt[(nb * 2 + h2) * 64 + lane];
                 }
 #pragma unroll
                 for (int cb = 0; cb < NC; ++cb) {
@@ -517,6 +531,68 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
                     o[cb][nb] = mfma_16x16x32(vf[1], pf[cb][1], o[cb][nb]);
                 }
             }
+        }
+    };
+
+    if constexpr (LDSP) {
+        // Many rows, pages through LDS: the workgroup's four waves (one head, 64 NC rows) bring every page they need
+        // between them into LDS once, straight from memory and a page ahead of the one being multiplied, in two
+        // buffers that take turns; a wave multiplies the pages its own rows see.
+        const int tbl = M.table_in_lds ? (A.bias_len + 3) / 4 * 4 : 0;         // floats in front of the pages
+        lds_u32x4* pages = (lds_u32x4*)(lds + tbl);
+        const int n_k = 4 * ksl, n_v = (vd / 16) * 2, buf_tiles = n_k + n_v;
+        const int g_lo = W > 0 ? max(0, wg_first - W + 1) : 0;
+        const int g_first = g_lo / AGAVE_PAGE;
+        const int g_kept = min(g_first, (keep + AGAVE_PAGE - 1) / AGAVE_PAGE);
+        const int g_n = g_kept + wg_last / AGAVE_PAGE - g_first + 1;
+        auto page_at = [&](int gi, int& pi) -> long {
+            pi = gi < g_kept ? gi : g_first + gi - g_kept;
+            const int col = page_col(pi, pbase, A.head);
+            const long pg = (col >= 0 && col < A.width) ? A.table[(size_t)b * A.width + col] : -1;
+            return pg < A.n_pages ? pg : -1;
+        };
+        auto fetch = [&](int gi, int buf) {
+            int pi;
+            const long pg = page_at(gi, pi);
+            if (pg < 0) return;
+            const uint4* ksrc = (const uint4*)A.k_pages + ((size_t)pg * nkv + kvh) * (size_t)n_k * 64;
+            const uint4* vsrc = (const uint4*)A.v_pages + ((size_t)pg * nkv + kvh) * (size_t)n_v * 64;
+            for (int ti = w; ti < buf_tiles; ti += 4) {
+                const uint4* src = ti < n_k ? ksrc + (size_t)ti * 64 : vsrc + (size_t)(ti - n_k) * 64;
+                lds_u32x4* dst = pages + ((size_t)buf * buf_tiles + ti) * 64;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + lane),
+                                                 (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+            }
+        };
+        fetch(0, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        for (int gi = 0; gi < g_n; ++gi) {
+            const int buf = gi & 1;
+            if (gi + 1 < g_n) fetch(gi + 1, buf ^ 1);
+            int pi;
+            const long pg = page_at(gi, pi);
+            const bool mine = wave_on && pg >= 0 && pi <= pmax / AGAVE_PAGE && (pi >= first_win || pi * AGAVE_PAGE < keep);
+            if (mine) {
+                const lds_u32x4* kl = pages + (size_t)buf * buf_tiles * 64;
+                page(pi, kl, kl + (size_t)n_k * 64);
+            }
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
+        if (!wave_on) return;
+    } else {
+        int idx = M.one_row ? w : 0;
+        long pg = page_of(idx);
+        for (; idx < n_pg; idx += stride) {
+            const long pg_next = page_of(idx + stride);         // asked for now, used in the next turn
+            const long pg_now = pg;
+            pg = pg_next;
+            if (pg_now < 0) continue;
+            const int pi = idx < n_kept ? idx : first_win + idx - n_kept;
+            const u32x4_t* kt = (const u32x4_t*)A.k_pages + ((size_t)pg_now * nkv + kvh) * (size_t)ksl * 4 * 64;
+            const u32x4_t* vt = (const u32x4_t*)A.v_pages + ((size_t)pg_now * nkv + kvh) * (size_t)(vd / 16) * 2 * 64;
+            page(pi, kt, vt);
         }
     }
     // the columns' sums over the four lane groups
@@ -547,7 +623,7 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
             const float m2 = other[c], l2 = other[16 + c];
             if (m2 == -INFINITY) continue;                      // (per lane: that wave saw nothing for my column)
             const float m_new = fmaxf(m[0], m2);
-            const float a1 = m[0] == -INFINITY ? 0.f : __expf(m[0] - m_new), a2 = __expf(m2 - m_new);
+            const float a1 = m[0] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[0] - m_new), a2 = __builtin_amdgcn_exp2f(m2 - m_new);
             l[0] = l[0] * a1 + l2 * a2;
             m[0] = m_new;
 #pragma unroll
@@ -582,22 +658,31 @@ __global__ __launch_bounds__(512) void attn_biased_mfma_kernel(BiasedArgs A, Mfm
 }
 
 template <int KS, int VB>
-static void launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid, int threads, int nc, size_t lds_bytes,
-                               hipStream_t stream) {
+static int launch_biased_mfma(const BiasedArgs& A, const MfmaMode& M, dim3 grid, int threads, int nc, size_t lds_bytes,
+                              hipStream_t stream) {
     if (nc == 2) {
-        if constexpr (VB <= 8)
-            attn_biased_mfma_kernel<KS, VB, 2><<<grid, threads, lds_bytes, stream>>>(A, M);
+        if constexpr (VB <= 8) {
+            static bool raised = false;             // (the two page buffers and the table may need more LDS than a kernel gets unasked)
+            if (!raised) {
+                AGAVE_CHECK(hipFuncSetAttribute((const void*)attn_biased_mfma_kernel<KS, VB, 2, true>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) == hipSuccess,
+                            "attn_biased_mfma: cannot raise the LDS allowance");
+                raised = true;
+            }
+            attn_biased_mfma_kernel<KS, VB, 2, true><<<grid, threads, lds_bytes, stream>>>(A, M);
+        }
     } else {
-        attn_biased_mfma_kernel<KS, VB, 1><<<grid, threads, lds_bytes, stream>>>(A, M);
+        attn_biased_mfma_kernel<KS, VB, 1, false><<<grid, threads, lds_bytes, stream>>>(A, M);
     }
+    return 0;
 }
 
 #define BIASED_VB(KS_)                                                                                   \
     switch (vb) {                                                                                        \
-        case 2: launch_biased_mfma<KS_, 2>(A, M, grid, threads, nc, lds_bytes, stream); break;           \
-        case 4: launch_biased_mfma<KS_, 4>(A, M, grid, threads, nc, lds_bytes, stream); break;           \
-        case 8: launch_biased_mfma<KS_, 8>(A, M, grid, threads, nc, lds_bytes, stream); break;           \
-        default: launch_biased_mfma<KS_, 16>(A, M, grid, threads, nc, lds_bytes, stream); break;         \
+        case 2: rc = launch_biased_mfma<KS_, 2>(A, M, grid, threads, nc, lds_bytes, stream); break;      \
+        case 4: rc = launch_biased_mfma<KS_, 4>(A, M, grid, threads, nc, lds_bytes, stream); break;      \
+        case 8: rc = launch_biased_mfma<KS_, 8>(A, M, grid, threads, nc, lds_bytes, stream); break;      \
+        default: rc = launch_biased_mfma<KS_, 16>(A, M, grid, threads, nc, lds_bytes, stream); break;    \
     }
 
 // 1 if the matrix-core kernel takes these sizes (the caller then may call it), else 0
@@ -637,20 +722,30 @@ extern "C" int agave_attn_biased_mfma(const void* q, long ldq, void* out, long l
         lds_bytes = (size_t)(nw - 1) * (vb * 16 * 16 + 32) * sizeof(float);
     } else {
         // 32 rows a wave where the step is long enough to fill the chip that way and the registers allow
+        // (then the workgroup's waves share a head's pages through LDS)
         nc = (vb <= 8 && (long)((max_rows + 127) / 128) * n_seqs * nh >= 256) ? 2 : 1;
-        grid = dim3((max_rows + 64 * nc - 1) / (64 * nc), n_seqs, nh);
-        AGAVE_CHECK(grid.y <= 65535 && grid.z <= 65535, "attn_biased_mfma: too many sequences or heads for the grid");
         if (bias_mode == 2 && bias_len <= 8192) {
             M.table_in_lds = 1;
-            lds_bytes = (size_t)bias_len * sizeof(float);
+            lds_bytes = (size_t)((bias_len + 3) / 4 * 4) * sizeof(float);
         }
+        if (nc == 2) {
+            const size_t page_bytes = (size_t)(4 * ((hd + 31) / 32) + (vd / 16) * 2) * 1024;
+            if (lds_bytes + 2 * page_bytes <= 144 * 1024)
+                lds_bytes += 2 * page_bytes;
+            else
+                nc = 1;
+        }
+        grid = dim3((max_rows + 64 * nc - 1) / (64 * nc), n_seqs, nh);
+        AGAVE_CHECK(grid.y <= 65535 && grid.z <= 65535, "attn_biased_mfma: too many sequences or heads for the grid");
     }
+    int rc = 0;
     switch (ks) {
         case 1: BIASED_VB(1); break;
         case 2: BIASED_VB(2); break;
         case 4: BIASED_VB(4); break;
         default: BIASED_VB(8); break;
     }
+    if (rc) return rc;
     AGAVE_LAUNCH_CHECK("attn_biased_mfma");
     return 0;
 }

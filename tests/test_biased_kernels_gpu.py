@@ -146,6 +146,23 @@ def test_attention_whole_in_pieces_and_token_by_token(shape, dtype):
         close(c.run(cuts(T, 180, 1), dtype), ref, dtype, f"{shape} on the plain kernel")
 
 
+@pytest.mark.parametrize("shape", [
+    (40, 4, 64, 64, 200, 70, "table", True, True),        # a window, two kept pages, sinks and a gate
+    (40, 2, 32, 48, None, 0, "slopes", False, False),     # every earlier key
+    (36, 36, 96, 16, 130, 0, "none", True, False),        # a head size that fills its last step in part
+])
+def test_long_prompts_share_pages_through_lds(shape):
+    """Steps long enough that the matrix-core kernel takes 32 rows a wave and brings the pages into LDS once for a
+    workgroup's four waves: a whole prompt, and a long piece behind a short one (the window reaches back into pages
+    of the earlier step, and the kept pages are not the window's)."""
+    T = 1100
+    c = Case(*shape, T=T, seed=7)
+    c.rounded(torch.bfloat16)
+    ref = c.plain()
+    close(c.run(cuts(T, T, 1), torch.bfloat16), ref, torch.bfloat16, f"{shape} whole")
+    close(c.run([(0, 230), (230, T)], torch.bfloat16), ref, torch.bfloat16, f"{shape} 230 + 870")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_a_batch_against_each_alone_and_slots_and_pages_used_again(dtype):
     from agave_amd.ops import attention_biased as A
