@@ -458,8 +458,13 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int c = lane & 15, g = lane >> 4;
     const int row0 = blockIdx.x * 16 * MI;
-    const int col0 = blockIdx.y * (64 * NJ) + w * (16 * NJ);
-    if (col0 >= n_out) return;
+    // A tile of 16 rows (MI == 1) streams its weights once: its four waves take the same 16 NJ columns and a quarter of
+    // K each, so that a wave's chain of loads is a quarter as long, and wave 0 adds the four sums through LDS.
+    constexpr bool KSPLIT = MI == 1;
+    const int col0 = KSPLIT ? blockIdx.y * (16 * NJ) : blockIdx.y * (64 * NJ) + w * (16 * NJ);
+    if (col0 >= n_out) return;                                  // (the whole workgroup where the waves split K)
+    const int k_share = KSPLIT ? ((K + 127) / 128) * 32 : K;    // whole steps of 32
+    const int k_begin = KSPLIT ? min(K, w * k_share) : 0, k_end = KSPLIT ? min(K, k_begin + k_share) : K;
     // A rows: 16 i + c of the tile
     const bf16* arow[MI];
 #pragma unroll
@@ -494,12 +499,12 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
             acc0[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             if (GATED) acc1[i][GATED ? j : 0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
-    int k_done = 0;
+    int k_done = k_begin;
     if constexpr (MI == 1) {
         // a tile of 16 rows streams its weights once and waits for memory, not for the matrix cores: the loads of
         // eight steps are asked for before the first is used
         constexpr int U = 8;
-        for (; k_done + 32 * U <= K; k_done += 32 * U) {
+        for (; k_done + 32 * U <= k_end; k_done += 32 * U) {
             frag16 a[U], bw0[U][NJ], bw1[U][NJ];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -520,7 +525,7 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
                 }
         }
     }
-    for (int k0 = k_done; k0 < K; k0 += 32) {
+    for (int k0 = k_done; k0 < k_end; k0 += 32) {
         // (loads without conditions, from inside the row; a lane past the row's end reads its start and is emptied)
         const bool in = k0 + 8 * g < K;
         const int at = in ? k0 : -8 * g;
@@ -544,6 +549,29 @@ __global__ __launch_bounds__(256) void routed_product_mfma_kernel(const bf16* __
                 acc0[i][j] = mfma_16x16x32(a[i], bw0[j], acc0[i][j]);
                 if (GATED) acc1[i][GATED ? j : 0] = mfma_16x16x32(a[i], bw1[j], acc1[i][GATED ? j : 0]);
             }
+    }
+    if constexpr (KSPLIT) {
+        __shared__ float part[3][2][NJ][256];
+        if (w > 0) {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    part[w - 1][0][j][e4 * 64 + lane] = acc0[0][j][e4];
+                    if (GATED) part[w - 1][1][j][e4 * 64 + lane] = acc1[0][GATED ? j : 0][e4];
+                }
+        }
+        __syncthreads();
+        if (w > 0) return;
+#pragma unroll
+        for (int ow = 0; ow < 3; ++ow)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    acc0[0][j][e4] += part[ow][0][j][e4 * 64 + lane];
+                    if (GATED) acc1[0][GATED ? j : 0][e4] += part[ow][1][j][e4 * 64 + lane];
+                }
     }
     // D[i][j]: lane holds rows 4 g + e4 of the row block, column c of the column block
 #pragma unroll
@@ -577,9 +605,9 @@ extern "C" int agave_routed_experts_mfma(const void* x, long ldx, const int* sor
     AGAVE_CHECK(x && sorted_pair && tile_expert && wg && wu && wd && act_rows && y, "routed_experts_mfma: null buffer");
     AGAVE_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)wg % 16) == 0 && ((uintptr_t)wu % 16) == 0 && ((uintptr_t)wd % 16) == 0 &&
                 ((uintptr_t)act_rows % 16) == 0, "routed_experts_mfma: buffers must be aligned to 16 bytes");
-    // tiles of 64 rows take 64 columns a wave (an operand that was loaded serves more multiplications), tiles of
-    // 16 rows, which stream their weights once, 16 (more workgroups, each with many loads in flight)
-    const int cols = TM == 64 ? 256 : 64;
+    // tiles of 64 rows take 64 columns a wave (an operand that was loaded serves more multiplications); a tile of
+    // 16 rows, which streams its weights once, takes 16 columns a workgroup, whose waves share K
+    const int cols = TM == 64 ? 256 : 16;
     const dim3 g1(max_tiles, (ff + cols - 1) / cols), g2(max_tiles, (hidden + cols - 1) / cols);
     AGAVE_CHECK(g1.y <= 65535 && g2.y <= 65535, "routed_experts_mfma: too many columns for the grid");
     if (TM == 64) {
