@@ -217,7 +217,7 @@ def one_key_stands_out(c, j0, marker):
     c.v[j0, :, :] = marker
 
 
-@pytest.mark.parametrize("window, keep", [(72, 6), (64, 1), (100, 64), (129, 65), (48, 0)])
+@pytest.mark.parametrize("window, keep", [(75, 7), (64, 1), (100, 64), (129, 65), (48, 0)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_a_dominant_key_just_inside_and_just_outside(window, keep, dtype):
     """The key is seen (the output is its value) up to the window's last query and not from the next on; a key among

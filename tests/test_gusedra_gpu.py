@@ -17,6 +17,12 @@ import plain_gusedra as P
 
 pytestmark = pytest.mark.gpu
 
+def reading(layer, source):
+    """The layer without keys and values of its own, reading those of layer ``source``."""
+    layer["mixer"]["kv_from"] = source
+    return layer
+
+
 CONFIGS = {
     # both mixers, grouped heads, values wider and narrower than keys, windows that are no multiples of a page and
     # differ from layer to layer, a reader with a wider window than the layer it reads, both feed-forwards
@@ -32,10 +38,19 @@ CONFIGS = {
         P.attention_layer(5, 1, 20, 12, None, mlp=P.moe(3, 0, 1, 1, 1, 1.0, 30)),
         P.attention2_layer(3, 3, 12, 20, None, 0, 300, mlp=None, buckets=20),
         P.attention_layer(5, 1, 20, 12, 17, kv_from=0, mlp=P.dense(50))], vocab=97, width=60, residual_mult=1.0),
+    # readers of the other kind than their source: slopes and sinks over the keys of a layer with a learned bias and kept
+    # positions (the pages then serve the reader's wider window and keep the source's first positions), and the reverse;
+    # a single layer of each kind without a feed-forward at the end; one router output more than experts, all chosen
+    "cross": lambda: P.config([
+        P.attention2_layer(4, 2, 16, 32, 40, 5, 64, mlp=P.moe(3, 1, 4, 1, 1, 1.0, 16), buckets=10),
+        P.attention_layer(6, 2, 16, 32, 60, kv_from=0, mlp=P.dense(48)),
+        P.attention_layer(2, 2, 32, 16, 100, mlp=None),
+        reading(P.attention2_layer(4, 2, 32, 16, 30, 70, 200, mlp=None, buckets=14), 2),
+    ], vocab=77, width=48, eps=1e-3, residual_mult=1.5),
     # sizes the matrix cores take, several pages of kept positions, everything a multiple of 16
     "even": lambda: P.config([
         P.attention2_layer(8, 2, 64, 64, 128, 130, 500, mlp=P.moe(8, 0, 2, 4, 2, 2.5, 64, shared_ff=64), buckets=32),
-        P.attention_layer(4, 4, 32, 64, 96, mlp=P.dense(256))], vocab=256, width=128, residual_mult=0.5),
+        P.attention_layer(4, 4, 32, 64, 96, mlp=P.dense(256))], vocab=256, width=128, residual_mult=0.6),
 }
 
 
