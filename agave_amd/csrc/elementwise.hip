@@ -369,6 +369,126 @@ __global__ void residual_layernorm_kernel(float* __restrict__ h, const T* __rest
     }
 }
 
+// The same with the row in registers, four neighbours a thread and chunk (one read of every input, one write of every
+// output, every load asked for before anything is used): for rows of up to threads * 4 * VPT elements whose pointers
+// allow 4-wide accesses.  A chunk past the row's end reads the row's start and is left out of the sums and the stores.
+template <typename T, int VPT>
+__global__ void residual_layernorm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
+                                               long part_stride, const float* __restrict__ post_w,
+                                               const float* __restrict__ post_b, float post_eps, T* __restrict__ out, long ldo,
+                                               const float* __restrict__ pre_w, const float* __restrict__ pre_b, float pre_eps,
+                                               const int* __restrict__ rows, int e, const float* __restrict__ h_src) {
+    __shared__ float red[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    float* hr = h + (size_t)r * e;
+    const float* hs = h_src ? h_src + (size_t)r * e : hr;
+    bool in[VPT];
+    int at[VPT];
+    float4 bv[VPT], hv[VPT], w1[VPT], b1[VPT], w2[VPT], b2[VPT];
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int c = (threadIdx.x + k * blockDim.x) * 4;
+        in[k] = c < e;
+        at[k] = in[k] ? c : 0;
+        hv[k] = *reinterpret_cast<const float4*>(hs + at[k]);
+        bv[k] = zero;
+        if (branch) {
+            if (n_parts == 0) {
+                bv[k] = load4(branch + (size_t)r * ldb + at[k]);
+            } else {
+                const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb + at[k];
+                for (int p = 0; p < n_parts; ++p) {
+                    const float4 v = *reinterpret_cast<const float4*>(parts + (size_t)p * part_stride);
+                    bv[k].x += v.x; bv[k].y += v.y; bv[k].z += v.z; bv[k].w += v.w;
+                }
+            }
+        }
+        w1[k] = post_w ? *reinterpret_cast<const float4*>(post_w + at[k]) : zero;
+        b1[k] = post_b ? *reinterpret_cast<const float4*>(post_b + at[k]) : zero;
+        w2[k] = pre_w ? *reinterpret_cast<const float4*>(pre_w + at[k]) : zero;
+        b2[k] = pre_b ? *reinterpret_cast<const float4*>(pre_b + at[k]) : zero;
+    }
+    auto mean_inv = [&](const float4* v, float eps, float& mean, float& inv) {
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < VPT; ++k)
+            if (in[k]) sum += v[k].x + v[k].y + v[k].z + v[k].w;
+        mean = block_sum(sum, red) / (float)e;          // (divided, not multiplied by a rounded 1/e: a constant row has mean = its value)
+        float sq = 0.f;
+#pragma unroll
+        for (int k = 0; k < VPT; ++k)
+            if (in[k]) {
+                const float dx = v[k].x - mean, dy = v[k].y - mean, dz = v[k].z - mean, dw = v[k].w - mean;
+                sq += dx * dx + dy * dy + dz * dz + dw * dw;
+            }
+        inv = 1.0f / sqrtf(block_sum(sq, red) / (float)e + eps);
+    };
+    if (branch) {
+        float mean = 0.f, inv = 1.f;
+        if (post_w) mean_inv(bv, post_eps, mean, inv);
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            float4 y = bv[k];
+            if (post_w) {
+                y.x = (y.x - mean) * inv * w1[k].x + b1[k].x;
+                y.y = (y.y - mean) * inv * w1[k].y + b1[k].y;
+                y.z = (y.z - mean) * inv * w1[k].z + b1[k].z;
+                y.w = (y.w - mean) * inv * w1[k].w + b1[k].w;
+            }
+            hv[k].x += y.x; hv[k].y += y.y; hv[k].z += y.z; hv[k].w += y.w;
+            if (in[k]) *reinterpret_cast<float4*>(hr + at[k]) = hv[k];
+        }
+    } else if (h_src) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k)
+            if (in[k]) *reinterpret_cast<float4*>(hr + at[k]) = hv[k];
+    }
+    if (out) {
+        float mean, inv;
+        mean_inv(hv, pre_eps, mean, inv);
+        T* o = out + (size_t)i * ldo;
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            float4 y;
+            y.x = (hv[k].x - mean) * inv * w2[k].x + b2[k].x;
+            y.y = (hv[k].y - mean) * inv * w2[k].y + b2[k].y;
+            y.z = (hv[k].z - mean) * inv * w2[k].z + b2[k].z;
+            y.w = (hv[k].w - mean) * inv * w2[k].w + b2[k].w;
+            if (in[k]) store4(o + at[k], y);
+        }
+    }
+}
+
+template <typename T>
+static bool launch_residual_layernorm_fast(float* h, const void* branch, long ldb, int n_parts, long part_stride,
+                                           const float* post_w, const float* post_b, float post_eps, void* out, long ldo,
+                                           const float* pre_w, const float* pre_b, float pre_eps, const int* rows, int n_rows,
+                                           int e, const float* h_src, hipStream_t stream) {
+    const size_t elem = n_parts ? sizeof(float) : sizeof(T);
+    auto a16 = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    const bool ok = e % 4 == 0 && e <= 8192 && a16(h) && a16(h_src) && a16(post_w) && a16(post_b) && a16(pre_w) && a16(pre_b) &&
+                    (!branch || (((uintptr_t)branch % (4 * elem)) == 0 && ldb % 4 == 0 && part_stride % 4 == 0)) &&
+                    (!out || (((uintptr_t)out % (4 * sizeof(T))) == 0 && ldo % 4 == 0));
+    if (!ok) return false;
+    const int threads = e <= 256 ? 64 : (e <= 4096 ? 256 : 512);
+    const int vpt = (e + threads * 4 - 1) / (threads * 4);
+#define LN_FAST(V)                                                                                                       \
+    residual_layernorm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride, \
+                                                                        post_w, post_b, post_eps, (T*)out, ldo, pre_w,   \
+                                                                        pre_b, pre_eps, rows, e, h_src)
+    switch (vpt) {
+        case 1: LN_FAST(1); break;
+        case 2: LN_FAST(2); break;
+        case 3: LN_FAST(3); break;
+        case 4: LN_FAST(4); break;
+        default: return false;
+    }
+#undef LN_FAST
+    return true;
+}
+
 // The arguments are residual_norm's, with a bias beside each weight (null: none).
 extern "C" int agave_residual_layernorm(int dtype, float* h, const void* branch, long ldb, int n_parts, long part_stride,
                                         const float* post_w, const float* post_b, float post_eps, void* out, long ldo,
@@ -385,7 +505,12 @@ extern "C" int agave_residual_layernorm(int dtype, float* h, const void* branch,
     if (n_rows == 0 || (!branch && !out && !h_src)) return 0;
     const int threads = e >= 2048 ? 512 : (e >= 512 ? 256 : 64);
     const size_t lds = (size_t)e * sizeof(float);
-    if (dtype == AGAVE_F32)
+    if (dtype == AGAVE_F32 && launch_residual_layernorm_fast<float>(h, branch, ldb, n_parts, part_stride, post_w, post_b, post_eps,
+                                                                   out, ldo, pre_w, pre_b, pre_eps, rows, n_rows, e, h_src, stream)) {
+    } else if (dtype == AGAVE_BF16 && launch_residual_layernorm_fast<bf16>(h, branch, ldb, n_parts, part_stride, post_w, post_b,
+                                                                          post_eps, out, ldo, pre_w, pre_b, pre_eps, rows, n_rows,
+                                                                          e, h_src, stream)) {
+    } else if (dtype == AGAVE_F32)
         residual_layernorm_kernel<float><<<n_rows, threads, lds, stream>>>(h, (const float*)branch, ldb, n_parts, part_stride, post_w,
                                                                            post_b, post_eps, (float*)out, ldo, pre_w, pre_b,
                                                                            pre_eps, rows, e, h_src);

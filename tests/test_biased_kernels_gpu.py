@@ -263,7 +263,7 @@ def test_the_sink_takes_its_share_and_the_bias_is_not_scaled():
 
 
 # ---------------------------------------------------------------- layer norm around the residual stream
-@pytest.mark.parametrize("e", [32, 257, 1000, 4096])
+@pytest.mark.parametrize("e", [32, 257, 1000, 4096, 6000, 9000])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_residual_layernorm(e, dtype):
     from agave_amd.ops import kernels as K
