@@ -91,10 +91,9 @@ extern "C" int agave_route_topk(const float* z, long ldz, const float* correctio
 }
 
 // ------------------------------------------------------------------ router product and choice in one kernel
-// A workgroup takes ROUTE_ROWS tokens: its waves share the router's outputs (a wave per output in turn, the lanes
+// A workgroup takes RR tokens: its waves share the router's outputs (a wave per output in turn, the lanes
 // along the width, a weight row read once for all of the workgroup's tokens), the logits wait in LDS, and one
 // thread per token then chooses as route_topk_kernel does.  The router matrix is 32-bit; the rows may be bfloat16.
-#define ROUTE_ROWS 8
 // eight neighbours along the width as floats (16 bytes of bfloat16, 32 of float)
 __device__ __forceinline__ void load8(const bf16* p, float* v) {
     const uint4 u = *reinterpret_cast<const uint4*>(p);
@@ -113,29 +112,31 @@ __device__ __forceinline__ void load8(const float* p, float* v) {
 // WIDE: the width is a multiple of 8 and the rows are aligned, so a lane takes eight neighbours at a time (a
 // fraction of the loads, many of them in flight); otherwise element by element.  The workgroup's waves (4, or 16
 // where few tokens leave the chip idle) take the outputs in turn.
-template <typename T, bool WIDE>
+// RR tokens a workgroup: eight where there are many, one where few tokens would leave the chip idle (a wave then holds
+// a whole row's share of loads in flight at once).
+template <typename T, bool WIDE, int RR>
 __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ router,
                                                           const float* __restrict__ correction, int N, int K, int R, int groups,
                                                           int keep, int top, float scale, int* __restrict__ choice,
                                                           float* __restrict__ weight) {
-    extern __shared__ float zs[];                      // [ROUTE_ROWS][R], then the corrections [R]
+    extern __shared__ float zs[];                      // [RR][R], then the corrections [R]
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    float* corr = zs + ROUTE_ROWS * R;                 // (read many times by the one thread that chooses: from LDS, not memory)
+    float* corr = zs + RR * R;                 // (read many times by the one thread that chooses: from LDS, not memory)
     for (int e = threadIdx.x; e < R; e += blockDim.x) corr[e] = correction ? correction[e] : 0.f;
-    const int t0 = blockIdx.x * ROUTE_ROWS;
-    const int rows = min(ROUTE_ROWS, N - t0);
+    const int t0 = blockIdx.x * RR;
+    const int rows = min(RR, N - t0);
     for (int r = w; r < R; r += nw) {
         const float* wr = router + (size_t)r * K;
-        float acc[ROUTE_ROWS];
+        float acc[RR];
 #pragma unroll
-        for (int i = 0; i < ROUTE_ROWS; ++i) acc[i] = 0.f;
+        for (int i = 0; i < RR; ++i) acc[i] = 0.f;
         if (WIDE) {
-#pragma unroll 2
+#pragma unroll(RR == 1 ? 4 : 2)
             for (int k = 8 * lane; k < K; k += 512) {
                 float wk[8];
                 load8(wr + k, wk);
 #pragma unroll
-                for (int i = 0; i < ROUTE_ROWS; ++i) {
+                for (int i = 0; i < RR; ++i) {
                     const int t = t0 + (i < rows ? i : 0);
                     float xv[8];
                     load8(x + (size_t)t * ldx + k, xv);
@@ -147,14 +148,14 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
             for (int k = lane; k < K; k += 64) {
                 const float wk = wr[k];
 #pragma unroll
-                for (int i = 0; i < ROUTE_ROWS; ++i) {
+                for (int i = 0; i < RR; ++i) {
                     const int t = t0 + (i < rows ? i : 0);
                     acc[i] = fmaf(ld(x + (size_t)t * ldx + k), wk, acc[i]);
                 }
             }
         }
 #pragma unroll
-        for (int i = 0; i < ROUTE_ROWS; ++i) {
+        for (int i = 0; i < RR; ++i) {
             const float sum = wave_sum(acc[i]);
             if (lane == 0) zs[i * R + r] = sum;
         }
@@ -192,6 +193,8 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
             }
         }
         // the `top` best of what is open; what was chosen is marked in the row's sign (s >= 0)
+        int my_choice = 0;
+        float my_weight = 0.f;
         for (int r = 0; r < top; ++r) {
             float best_v = -INFINITY;
             int best = -1;
@@ -208,14 +211,20 @@ __global__ __launch_bounds__(1024) void route_rows_kernel(const T* __restrict__ 
             const int chosen = (int)(-wave_max((best >= 0 && best_v == top_v) ? -(float)best : -INFINITY));
             // (top <= open outputs is checked on the host, so some lane has a candidate)
             const float s_chosen = sr[chosen];
-            if (lane == 0) {
-                choice[(size_t)t * top + r] = chosen;
-                weight[(size_t)t * top + r] = s_chosen * scale;
-                sr[chosen] = -1.0f - s_chosen;
+            if ((r & 63) == lane) {             // lane r keeps round r's result; the results leave in one store at the end
+                my_choice = chosen;
+                my_weight = s_chosen * scale;
             }
+            if (lane == 0) sr[chosen] = -1.0f - s_chosen;
+            // (a wave's LDS accesses happen in the order they were issued: the next round's reads see this write)
             __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if ((r & 63) == 63 || r == top - 1) {
+                const int at = (r & ~63) + lane;
+                if (at <= r) {
+                    choice[(size_t)t * top + at] = my_choice;
+                    weight[(size_t)t * top + at] = my_weight;
+                }
+            }
         }
     }
 }
@@ -229,26 +238,22 @@ extern "C" int agave_route_rows(int dtype, const void* x, long ldx, const float*
     AGAVE_CHECK(top > 0 && top <= keep * (R / groups), "route_rows: %d chosen of %d that are open", top, keep * (R / groups));
     AGAVE_CHECK(x && router && choice && weight && ldx >= K, "route_rows: bad buffers");
     if (N == 0) return 0;
-    const int blocks = (N + ROUTE_ROWS - 1) / ROUTE_ROWS;
-    const size_t lds = (size_t)(ROUTE_ROWS + 1) * R * sizeof(float);
-    const int threads = blocks < 128 ? 1024 : 256;
     const bool wide = K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 32) == 0 && ((uintptr_t)router % 32) == 0;
-    if (dtype == AGAVE_F32) {
-        if (wide)
-            route_rows_kernel<float, true><<<blocks, threads, lds, stream>>>((const float*)x, ldx, router, correction, N, K, R, groups,
-                                                                             keep, top, scale, choice, weight);
-        else
-            route_rows_kernel<float, false><<<blocks, threads, lds, stream>>>((const float*)x, ldx, router, correction, N, K, R, groups,
-                                                                              keep, top, scale, choice, weight);
-    } else if (dtype == AGAVE_BF16) {
-        if (wide)
-            route_rows_kernel<bf16, true><<<blocks, threads, lds, stream>>>((const bf16*)x, ldx, router, correction, N, K, R, groups,
-                                                                            keep, top, scale, choice, weight);
-        else
-            route_rows_kernel<bf16, false><<<blocks, threads, lds, stream>>>((const bf16*)x, ldx, router, correction, N, K, R, groups,
-                                                                             keep, top, scale, choice, weight);
-    } else
-        AGAVE_CHECK(false, "route_rows: unknown dtype %d", dtype);
+    AGAVE_CHECK(dtype == AGAVE_F32 || dtype == AGAVE_BF16, "route_rows: unknown dtype %d", dtype);
+    const bool f32 = dtype == AGAVE_F32;
+    if (N <= 64) {
+        const size_t lds = (size_t)2 * R * sizeof(float);
+#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 1><<<N, 1024, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight)
+        if (f32 && wide) ROUTE_GO(float, true); else if (f32) ROUTE_GO(float, false); else if (wide) ROUTE_GO(bf16, true); else ROUTE_GO(bf16, false);
+#undef ROUTE_GO
+    } else {
+        const int blocks = (N + 7) / 8;
+        const size_t lds = (size_t)9 * R * sizeof(float);
+        const int threads = blocks <= 512 ? 1024 : 256;        // (more waves to share the outputs while they all fit the chip at once)
+#define ROUTE_GO(T_, W_) route_rows_kernel<T_, W_, 8><<<blocks, threads, lds, stream>>>((const T_*)x, ldx, router, correction, N, K, R, groups, keep, top, scale, choice, weight)
+        if (f32 && wide) ROUTE_GO(float, true); else if (f32) ROUTE_GO(float, false); else if (wide) ROUTE_GO(bf16, true); else ROUTE_GO(bf16, false);
+#undef ROUTE_GO
+    }
     AGAVE_LAUNCH_CHECK("route_rows");
     return 0;
 }
