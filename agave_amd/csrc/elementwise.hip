@@ -372,13 +372,27 @@ __global__ void residual_layernorm_kernel(float* __restrict__ h, const T* __rest
 // The same with the row in registers, four neighbours a thread and chunk (one read of every input, one write of every
 // output, every load asked for before anything is used): for rows of up to threads * 4 * VPT elements whose pointers
 // allow 4-wide accesses.  A chunk past the row's end reads the row's start and is left out of the sums and the stores.
-template <typename T, int VPT>
+// BR: 0 no branch, 1 a branch of rows, 2 a branch of 32-bit slices (known when the kernel is compiled, so that no load
+// stands under a condition: such a load is waited for on the spot, and the row would make a round trip to memory per
+// operand instead of one).  Weights and biases that are absent are read from the residual row instead and not used.
+template <typename T, int VPT, int BR>
 __global__ void residual_layernorm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
                                                long part_stride, const float* __restrict__ post_w,
                                                const float* __restrict__ post_b, float post_eps, T* __restrict__ out, long ldo,
                                                const float* __restrict__ pre_w, const float* __restrict__ pre_b, float pre_eps,
                                                const int* __restrict__ rows, int e, const float* __restrict__ h_src) {
-    __shared__ float red[16];
+    // four sums over the row, each with LDS places of its own: one barrier a sum (a place that is used again needs a
+    // second one to guard it, and this kernel's time is its chain of barriers)
+    __shared__ float red[4][16];
+    const int lane_ = threadIdx.x & 63, wave_ = threadIdx.x >> 6, n_waves = (blockDim.x + 63) >> 6;
+    auto row_sum = [&](float v, int which) {
+        v = wave_sum(v);
+        if (lane_ == 0) red[which][wave_] = v;
+        __syncthreads();
+        float r = 0.f;
+        for (int k = 0; k < n_waves; ++k) r += red[which][k];
+        return r;
+    };
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
     float* hr = h + (size_t)r * e;
@@ -394,28 +408,34 @@ __global__ void residual_layernorm_fast_kernel(float* __restrict__ h, const T* _
         at[k] = in[k] ? c : 0;
         hv[k] = *reinterpret_cast<const float4*>(hs + at[k]);
         bv[k] = zero;
-        if (branch) {
-            if (n_parts == 0) {
-                bv[k] = load4(branch + (size_t)r * ldb + at[k]);
-            } else {
-                const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb + at[k];
-                for (int p = 0; p < n_parts; ++p) {
-                    const float4 v = *reinterpret_cast<const float4*>(parts + (size_t)p * part_stride);
-                    bv[k].x += v.x; bv[k].y += v.y; bv[k].z += v.z; bv[k].w += v.w;
-                }
+        if (BR == 1) bv[k] = load4(branch + (size_t)r * ldb + at[k]);
+        w1[k] = *reinterpret_cast<const float4*>((post_w ? post_w : hs) + at[k]);
+        b1[k] = *reinterpret_cast<const float4*>((post_b ? post_b : hs) + at[k]);
+        w2[k] = *reinterpret_cast<const float4*>((pre_w ? pre_w : hs) + at[k]);
+        b2[k] = *reinterpret_cast<const float4*>((pre_b ? pre_b : hs) + at[k]);
+    }
+    if (BR == 2) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb + at[k];
+#pragma unroll 4
+            for (int p = 0; p < n_parts; ++p) {
+                const float4 v = *reinterpret_cast<const float4*>(parts + (size_t)p * part_stride);
+                bv[k].x += v.x; bv[k].y += v.y; bv[k].z += v.z; bv[k].w += v.w;
             }
         }
-        w1[k] = post_w ? *reinterpret_cast<const float4*>(post_w + at[k]) : zero;
-        b1[k] = post_b ? *reinterpret_cast<const float4*>(post_b + at[k]) : zero;
-        w2[k] = pre_w ? *reinterpret_cast<const float4*>(pre_w + at[k]) : zero;
-        b2[k] = pre_b ? *reinterpret_cast<const float4*>(pre_b + at[k]) : zero;
     }
-    auto mean_inv = [&](const float4* v, float eps, float& mean, float& inv) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        if (!post_b) b1[k] = zero;
+        if (!pre_b) b2[k] = zero;
+    }
+    auto mean_inv = [&](const float4* v, float eps, float& mean, float& inv, int which) {
         float sum = 0.f;
 #pragma unroll
         for (int k = 0; k < VPT; ++k)
             if (in[k]) sum += v[k].x + v[k].y + v[k].z + v[k].w;
-        mean = block_sum(sum, red) / (float)e;          // (divided, not multiplied by a rounded 1/e: a constant row has mean = its value)
+        mean = row_sum(sum, which) / (float)e;          // (divided, not multiplied by a rounded 1/e: a constant row has mean = its value)
         float sq = 0.f;
 #pragma unroll
         for (int k = 0; k < VPT; ++k)
@@ -423,11 +443,11 @@ __global__ void residual_layernorm_fast_kernel(float* __restrict__ h, const T* _
                 const float dx = v[k].x - mean, dy = v[k].y - mean, dz = v[k].z - mean, dw = v[k].w - mean;
                 sq += dx * dx + dy * dy + dz * dz + dw * dw;
             }
-        inv = 1.0f / sqrtf(block_sum(sq, red) / (float)e + eps);
+        inv = 1.0f / sqrtf(row_sum(sq, which + 1) / (float)e + eps);
     };
-    if (branch) {
+    if (BR != 0) {
         float mean = 0.f, inv = 1.f;
-        if (post_w) mean_inv(bv, post_eps, mean, inv);
+        if (post_w) mean_inv(bv, post_eps, mean, inv, 0);
 #pragma unroll
         for (int k = 0; k < VPT; ++k) {
             float4 y = bv[k];
@@ -447,7 +467,7 @@ __global__ void residual_layernorm_fast_kernel(float* __restrict__ h, const T* _
     }
     if (out) {
         float mean, inv;
-        mean_inv(hv, pre_eps, mean, inv);
+        mean_inv(hv, pre_eps, mean, inv, 2);
         T* o = out + (size_t)i * ldo;
 #pragma unroll
         for (int k = 0; k < VPT; ++k) {
@@ -474,10 +494,16 @@ static bool launch_residual_layernorm_fast(float* h, const void* branch, long ld
     if (!ok) return false;
     const int threads = e <= 256 ? 64 : (e <= 4096 ? 256 : 512);
     const int vpt = (e + threads * 4 - 1) / (threads * 4);
-#define LN_FAST(V)                                                                                                       \
-    residual_layernorm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride, \
-                                                                        post_w, post_b, post_eps, (T*)out, ldo, pre_w,   \
-                                                                        pre_b, pre_eps, rows, e, h_src)
+#define LN_GO(V, B)                                                                                                         \
+    residual_layernorm_fast_kernel<T, V, B><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride, \
+                                                                           post_w, post_b, post_eps, (T*)out, ldo, pre_w,   \
+                                                                           pre_b, pre_eps, rows, e, h_src)
+#define LN_FAST(V)                         \
+    do {                                   \
+        if (!branch) LN_GO(V, 0);          \
+        else if (n_parts == 0) LN_GO(V, 1);\
+        else LN_GO(V, 2);                  \
+    } while (0)
     switch (vpt) {
         case 1: LN_FAST(1); break;
         case 2: LN_FAST(2); break;
@@ -486,6 +512,7 @@ static bool launch_residual_layernorm_fast(float* h, const void* branch, long ld
         default: return false;
     }
 #undef LN_FAST
+#undef LN_GO
     return true;
 }
 

@@ -330,19 +330,23 @@ __global__ void routed_combine_kernel(const float* __restrict__ y, const int* __
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long)N * hidden) return;
     const int t = (int)(idx / hidden), c = (int)(idx % hidden);
+    // (no load under a per-lane condition: the input row's element is read once, an expert row's from a row that exists
+    // whatever the choice, and what does not count is left out afterwards)
+    const float xv = ld(x + (size_t)t * ldx + c);
+    const float sv = ld((shared ? shared : x) + (size_t)t * (shared ? lds : ldx) + c);
     float acc = 0.f;
+#pragma unroll 4
     for (int r = 0; r < top; ++r) {
         const int p = t * top + r;
         const int e = choice[p];
         const float w = weight[p];
-        if (e >= E) {
-            acc = fmaf(w, ld(x + (size_t)t * ldx + c), acc);
-        } else if (e >= 0) {
-            const int row = place ? place[p] : p;
-            acc = fmaf(w, y[(size_t)row * hidden + c], acc);
-        }
+        const bool expert = e >= 0 && e < E;
+        int row = place ? place[p] : p;
+        row = (expert && row >= 0) ? row : 0;
+        const float yv = y ? y[(size_t)row * hidden + c] : 0.f;
+        acc = fmaf(w, e >= E ? xv : (expert ? yv : 0.f), acc);
     }
-    if (shared) acc += ld(shared + (size_t)t * lds + c);
+    if (shared) acc += sv;
     st(out + (size_t)t * ldo + c, acc);
 }
 
