@@ -146,6 +146,19 @@ def test_attention_whole_in_pieces_and_token_by_token(shape, dtype):
         close(c.run(cuts(T, 180, 1), dtype), ref, dtype, f"{shape} on the plain kernel")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_table_too_long_for_lds_is_read_from_memory(dtype):
+    """A bias over distances up to 20,000: the table's row of a head does not fit the kernel's LDS allowance and is read
+    from memory, in short steps, in a long prompt (pages through LDS, the table not) and token by token."""
+    c = Case(40, 4, 32, 32, 600, 3, "table", False, False, T=1100, seed=11, buckets=24, D=20000)
+    assert c.bias.shape[1] > 8192
+    c.rounded(dtype)
+    ref = c.plain()
+    close(c.run(cuts(1100, 1100, 1), dtype), ref, dtype, "whole")
+    close(c.run(cuts(1100, 1000, 7), dtype), ref, dtype, "1,000 and pieces of 7")
+    close(c.run(cuts(1100, 1090, 1), dtype), ref, dtype, "the last ten one by one")
+
+
 @pytest.mark.parametrize("shape", [
     (40, 4, 64, 64, 200, 70, "table", True, True),        # a window, two kept pages, sinks and a gate
     (40, 2, 32, 48, None, 0, "slopes", False, False),     # every earlier key
