@@ -18,7 +18,8 @@
 // columns after them run from the oldest page the window reaches (base[b]) to the newest.
 //
 // Kernels: rows into the cache; a plain kernel (a workgroup per token and head, any sizes, both
-// element types); a matrix-core kernel for many query rows (bfloat16, sizes in steps of 16).
+// element types, either page order); a matrix-core kernel for prompts and for decode steps
+// (bfloat16, pages in operand order, keys in steps of 8 and values in steps of 16 up to 256).
 #include "common_impl.h"
 #include "mfma.h"
 #include <math.h>

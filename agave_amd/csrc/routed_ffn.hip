@@ -10,7 +10,7 @@
 //
 // A (token, slot) pair p = t * top + slot names one chosen output.  The plain kernels take the pairs
 // as they come (a wave per pair and output column).  The matrix-core kernels take them sorted by
-// expert, in tiles of 64 pairs that never span two experts (`route_sort` makes the list and the
+// expert, in tiles of 16 or 64 pairs that never span two experts (`route_sort` makes the list and the
 // tiles' table on the device, so a step's launches never depend on the choice).
 #include "common_impl.h"
 #include "mfma.h"
